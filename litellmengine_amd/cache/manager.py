@@ -1,0 +1,258 @@
+"""The cache manager: pages of keys and values with a block table per request,
+in groups, and slots of fixed-size per-request state.
+
+Reference: ModelPagedKVCache (src/engine/paged_kv_cache.cpp:18-105),
+BlockTableManager (src/engine/block_table_manager.cpp:17-274) and
+PagedKVCacheManager (src/engine/paged_kv_cache_manager.cpp:9-140).  Kept from
+it: one page id serves every layer of its group, all-or-nothing growth
+(:60-89), LIFO reuse, `token slot = table[pos / P] * P + pos % P` (:91-122),
+no zero-filling of reused pages (lengths say what is valid).  Different:
+ * block tables live on the device as one int32 matrix per group, row = request
+   slot; only new entries travel (the reference packs and uploads the whole
+   table per layer per step, src/ops/attention.cu:959-1020);
+ * cache layers with the same needs form a group with pages and tables of its
+   own; a group with a window gives pages back as soon as the window has
+   passed them;
+ * mixers may ask for fixed-size state rows, zeroed at admission.
+
+Pool layout of a group: [layer, page, 2 (K, V), kv_head, page_size, head_dim].
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..parts.base import KVCacheSpec, StateSpec
+from .page_pool import OutOfPages, PagePool
+
+
+class CacheGroup:
+    """Pages, pool and block tables of the cache layers that share one KVCacheSpec."""
+
+    def __init__(self, index: int, spec: KVCacheSpec, cache_ids: Sequence[int], page_size: int, num_pages: int,
+                 max_requests: int, max_pages_per_request: int, dtype: torch.dtype, device: torch.device):
+        self.index = index
+        self.spec = spec
+        self.cache_ids = list(cache_ids)
+        self.page_size = page_size
+        self.window = spec.window
+        self.pool = PagePool(num_pages)
+        self.max_pages_per_request = max_pages_per_request
+        self.kv = torch.zeros(
+            (len(self.cache_ids), num_pages, 2, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype, device=device
+        )
+        # per request slot: logical page -> physical page (-1 once the window has passed it)
+        self.tables: List[List[int]] = [[] for _ in range(max_requests)]
+        self.first_live: List[int] = [0] * max_requests
+        self.block_table = torch.full((max_requests, max_pages_per_request), -1, dtype=torch.int32, device=device)
+        self.pending: Dict[int, int] = {}  # flat index into block_table -> page, not yet on the device
+        self.slot_mapping: Optional[torch.Tensor] = None  # int32 [N] of the step being run
+
+    def pages_for(self, length: int) -> int:
+        return (length + self.page_size - 1) // self.page_size
+
+    def new_pages_needed(self, slot: int, new_len: int) -> int:
+        return max(0, self.pages_for(new_len) - len(self.tables[slot]))
+
+    def grow(self, slot: int, new_len: int) -> None:
+        need = self.new_pages_needed(slot, new_len)
+        if need == 0:
+            return
+        table = self.tables[slot]
+        if len(table) + need > self.max_pages_per_request:
+            raise OutOfPages(
+                f"a request may hold {self.max_pages_per_request} pages of {self.page_size} tokens; "
+                f"{new_len} tokens need {len(table) + need}"
+            )
+        for page in self.pool.allocate(need):
+            self.pending[slot * self.max_pages_per_request + len(table)] = page
+            table.append(page)
+
+    def trim(self, slot: int, length: int) -> None:
+        """Give back the pages that no later query can see: with a window w the
+        next query (position `length`) sees keys >= length - w + 1."""
+        if self.window is None:
+            return
+        first_needed = max(0, length - self.window + 1) // self.page_size
+        table = self.tables[slot]
+        first = self.first_live[slot]
+        if first_needed > first:
+            last = min(first_needed, len(table))
+            self.pool.release([table[i] for i in range(first, last)])
+            for i in range(first, last):
+                table[i] = -1
+            self.first_live[slot] = last
+
+    def release(self, slot: int) -> None:
+        table = self.tables[slot]
+        self.pool.release([p for p in table[self.first_live[slot]:]])
+        self.tables[slot] = []
+        self.first_live[slot] = 0
+
+    def token_slot(self, slot: int, pos: int) -> int:
+        page = self.tables[slot][pos // self.page_size]
+        if page < 0:
+            raise IndexError(f"position {pos} lies in a page that was given back")
+        return page * self.page_size + pos % self.page_size
+
+    def apply_table_updates(self, flat_index: torch.Tensor, pages: torch.Tensor) -> None:
+        """Write new table entries (int32 device arrays) into the device table."""
+        self.block_table.view(-1).index_copy_(0, flat_index.long(), pages)
+
+    def held_pages(self, slot: int) -> List[int]:
+        return [p for p in self.tables[slot] if p >= 0]
+
+
+@dataclasses.dataclass
+class LayerCache:
+    """What the mixer of one plan entry gets: the pages of its cache layer
+    [page, 2, kv_head, page_size, head_dim], its group (block table and the
+    step's slot mapping), whether it writes, and its state rows [slot, ...]."""
+
+    group: Optional[CacheGroup]
+    kv: Optional[torch.Tensor]
+    writes: bool
+    state: Optional[torch.Tensor]
+
+
+class CacheManager:
+    def __init__(self, model, *, page_size: int, num_pages: int, max_requests: int,
+                 max_pages_per_request: Optional[int] = None, dtype: torch.dtype, device):
+        """`model` is a models.decoder.DecoderLM (its plan and mixers say what is
+        needed); every group gets `num_pages` pages of `page_size` tokens."""
+        if page_size <= 0:
+            raise ValueError("--page-size must be positive")  # src/main.cpp:62-64
+        device = torch.device(device)
+        self.page_size = page_size
+        self.max_requests = max_requests
+        self.device = device
+        self.dtype = dtype
+        max_pages_per_request = max_pages_per_request or num_pages
+
+        by_spec: Dict[KVCacheSpec, List[int]] = {}
+        for cache_id, mixer in sorted(model.cache_layers().items()):
+            spec = mixer.cache_spec()
+            if spec is not None:
+                by_spec.setdefault(spec, []).append(cache_id)
+        self.groups: List[CacheGroup] = [
+            CacheGroup(g, spec, ids, page_size, num_pages, max_requests, max_pages_per_request, dtype, device)
+            for g, (spec, ids) in enumerate(by_spec.items())
+        ]
+        where: Dict[int, Tuple[CacheGroup, int]] = {}
+        for group in self.groups:
+            for n, cache_id in enumerate(group.cache_ids):
+                where[cache_id] = (group, n)
+
+        # state rows belong to a cache id too: every entry that names it shares them
+        self.states: Dict[int, torch.Tensor] = {}
+        self._layers: List[LayerCache] = []
+        for entry in model.plan:
+            mixer = model.blocks[entry.block].mixer
+            sspec: Optional[StateSpec] = mixer.state_spec()
+            if sspec is not None and entry.cache not in self.states:
+                self.states[entry.cache] = torch.zeros((max_requests,) + tuple(sspec.shape), dtype=sspec.dtype, device=device)
+            group, n = where.get(entry.cache, (None, 0))
+            self._layers.append(
+                LayerCache(group, None if group is None else group.kv[n], entry.writes, self.states.get(entry.cache))
+            )
+
+        self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
+        self._live = bytearray(max_requests)
+        self._length: List[int] = [0] * max_requests
+
+    # -- request slots -----------------------------------------------------------
+    @property
+    def num_free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def admit(self) -> int:
+        """A slot for a new request: empty tables, length 0, state rows zeroed."""
+        if not self._free_slots:
+            raise OutOfPages("no free request slot")
+        slot = self._free_slots.pop()
+        self._live[slot] = 1
+        self._length[slot] = 0
+        for state in self.states.values():
+            state[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        """Give back everything the request holds (pages of every group, its slot)."""
+        self._check_live(slot)
+        for group in self.groups:
+            group.release(slot)
+        self._live[slot] = 0
+        self._length[slot] = 0
+        self._free_slots.append(slot)
+
+    def is_live(self, slot: int) -> bool:
+        return 0 <= slot < self.max_requests and bool(self._live[slot])
+
+    def length(self, slot: int) -> int:
+        self._check_live(slot)
+        return self._length[slot]
+
+    def _check_live(self, slot: int) -> None:
+        if not self.is_live(slot):
+            raise ValueError(f"request slot {slot} is not in use")
+
+    # -- pages -----------------------------------------------------------------------
+    def can_extend(self, wants: Sequence[Tuple[int, int]]) -> bool:
+        """Would `extend_many(wants)` succeed?  wants = [(slot, new_len), ...]."""
+        for group in self.groups:
+            need = 0
+            for slot, new_len in wants:
+                n = group.new_pages_needed(slot, new_len)
+                if len(group.tables[slot]) + n > group.max_pages_per_request:
+                    return False
+                need += n
+            if need > group.pool.num_free:
+                return False
+        return True
+
+    def extend_many(self, wants: Sequence[Tuple[int, int]]) -> None:
+        """Make room for positions < new_len of every (slot, new_len): all or nothing."""
+        for slot, new_len in wants:
+            self._check_live(slot)
+            if new_len < self._length[slot]:
+                raise ValueError("a request cannot shrink")
+        if not self.can_extend(wants):
+            free = ", ".join(f"group {g.index}: {g.pool.num_free}" for g in self.groups)
+            raise OutOfPages(f"not enough free physical blocks for this step (free pages: {free})")
+        for group in self.groups:
+            for slot, new_len in wants:
+                group.grow(slot, new_len)
+
+    def extend(self, slot: int, new_len: int) -> None:
+        self.extend_many([(slot, new_len)])
+
+    def commit(self, slot: int, new_len: int) -> None:
+        """The positions < new_len are now written; windows move on."""
+        self._check_live(slot)
+        self._length[slot] = new_len
+        for group in self.groups:
+            group.trim(slot, new_len)
+
+    def free_pages(self) -> List[int]:
+        return [g.pool.num_free for g in self.groups]
+
+    def pages_needed(self, slot: Optional[int], new_len: int) -> List[int]:
+        """New pages per group that growing `slot` (None: a fresh request) to new_len takes."""
+        return [
+            g.pages_for(new_len) if slot is None else g.new_pages_needed(slot, new_len) for g in self.groups
+        ]
+
+    # -- what a step needs ---------------------------------------------------------------
+    def layer(self, plan_index: int) -> LayerCache:
+        return self._layers[plan_index]
+
+    def take_table_updates(self):
+        """[(group index, flat indices, pages)] of table entries not yet on the device."""
+        out = []
+        for g in self.groups:
+            if g.pending:
+                out.append((g.index, list(g.pending.keys()), list(g.pending.values())))
+                g.pending = {}
+        return out

@@ -1,0 +1,55 @@
+// Embedding row gather and SiLU-and-mul.
+// Counterparts in the reference: embedding_forward_kernel
+// (src/layers/embedding.cu:91-118) and silu_and_mul_kernel
+// (src/ops/silu_and_mul.cu:64-80); both are 32-bit only there.
+#include "common.h"
+
+LLE_DEFINE_ERROR_STRING()
+
+// out[n, :] = table[ids[n], :] as 32-bit (the residual stream is 32-bit in
+// every mode).  The host has checked 0 <= id < V.
+template <typename T>
+__global__ __launch_bounds__(256) void embedding_kernel(const int32_t* __restrict__ ids,
+                                                         const T* __restrict__ table,
+                                                         float* __restrict__ out, int H) {
+    const int64_t n = blockIdx.x;
+    const T* row = table + (int64_t)ids[n] * H;
+    float* o = out + n * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<T>(row[i]);
+}
+
+extern "C" int lle_embedding(const void* ids, const void* table, void* out, int N, int H, int dtype,
+                             hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (dtype == LLE_F32)
+        embedding_kernel<float><<<N, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, H);
+    else
+        embedding_kernel<bf16_t><<<N, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, H);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// gate_up [N, 2I] (gate columns first) -> out [N, I] = gate / (1 + exp(-gate)) * up, in 32-bit
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out,
+                                                        int64_t total, int I) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t n = idx / I;
+        const int i = (int)(idx - n * I);
+        const float g = to_f32<T>(gate_up[n * 2 * I + i]);
+        const float u = to_f32<T>(gate_up[n * 2 * I + I + i]);
+        out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    }
+}
+
+extern "C" int lle_silu_mul(const void* gate_up, void* out, int N, int I, int dtype, hipStream_t stream) {
+    const int64_t total = (int64_t)N * I;
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == LLE_F32)
+        silu_mul_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, total, I);
+    else
+        silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, total, I);
+    LLE_RETURN_LAUNCH_STATUS();
+}

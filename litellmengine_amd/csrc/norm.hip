@@ -1,0 +1,85 @@
+// RMSNorm fused with the residual add.
+// Reference counterparts: rms_norm_forward_kernel (src/layers/rms_norm.cu:97-141)
+// and add_fp32_kernel (src/ops/add.cu:16-27), two launches there.
+//
+//   h = hidden[row] (+ delta[row])          32-bit sum, the residual stream
+//   out[r] = h * rsqrt(mean(h^2) + eps) * w
+// With `rows == nullptr` row r is r and h is written back to `hidden`; with a
+// row list (the output head: only the wanted rows) nothing is written back.
+#include "common.h"
+
+LLE_DEFINE_ERROR_STRING()
+
+template <typename T>
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(float* __restrict__ hidden, const T* __restrict__ delta,
+                                                            const int32_t* __restrict__ rows,
+                                                            const void* __restrict__ weight, int weight_dtype,
+                                                            T* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    const int64_t row = rows ? (int64_t)rows[r] : r;
+    float* h = hidden + row * H;
+    const T* dl = delta ? delta + row * H : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = h[i];
+        if (dl) v += to_f32<T>(dl[i]);
+        if (!rows && dl) h[i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + r * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = h[i];
+        if (rows && dl) v += to_f32<T>(dl[i]);
+        o[i] = from_f32<T>(v * inv * load_as_f32(weight, i, weight_dtype));
+    }
+}
+
+extern "C" int lle_add_rmsnorm(void* hidden, const void* delta, const void* rows, const void* weight,
+                               int weight_dtype, void* out, int R, int H, float eps, int dtype,
+                               hipStream_t stream) {
+    if (R <= 0) return 0;
+    int threads = 256;
+    if (H > 2048) threads = 512;
+    if (H > 8192) threads = 1024;
+    if (dtype == LLE_F32)
+        add_rmsnorm_kernel<float><<<R, threads, 0, stream>>>((float*)hidden, (const float*)delta,
+                                                              (const int32_t*)rows, weight, weight_dtype,
+                                                              (float*)out, H, eps);
+    else
+        add_rmsnorm_kernel<bf16_t><<<R, threads, 0, stream>>>((float*)hidden, (const bf16_t*)delta,
+                                                               (const int32_t*)rows, weight, weight_dtype,
+                                                               (bf16_t*)out, H, eps);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// plain RMSNorm of activation rows x [R, H] of type T (no residual): out = norm(x) * w
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const void* __restrict__ weight,
+                                                       int weight_dtype, T* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    const T* xr = x + r * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = to_f32<T>(xr[i]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + r * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x)
+        o[i] = from_f32<T>(to_f32<T>(xr[i]) * inv * load_as_f32(weight, i, weight_dtype));
+}
+
+extern "C" int lle_rmsnorm(const void* x, const void* weight, int weight_dtype, void* out, int R, int H, float eps,
+                           int dtype, hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (dtype == LLE_F32)
+        rmsnorm_kernel<float><<<R, 256, 0, stream>>>((const float*)x, weight, weight_dtype, (float*)out, H, eps);
+    else
+        rmsnorm_kernel<bf16_t><<<R, 256, 0, stream>>>((const bf16_t*)x, weight, weight_dtype, (bf16_t*)out, H, eps);
+    LLE_RETURN_LAUNCH_STATUS();
+}

@@ -1,0 +1,245 @@
+"""Python face of the HIP kernels: checks operands on the host, then launches
+on the current stream.  Tensors are torch tensors on the GPU (torch is the
+allocator and the stream owner; the arithmetic is in `*.hip`).  There is no
+CPU path: without a GPU or without the compiled libraries these raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_L = ctypes.c_int64
+_F = ctypes.c_float
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, not {dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None) -> None:
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+
+
+class HipOps:
+    """The operations a model part may call.  One instance per process is enough."""
+
+    MAX_HEAD_DIM = 256
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("litellmengine_amd needs a GPU: its kernels have no CPU form")
+        self._fn = {}
+
+    # -- plumbing ---------------------------------------------------------
+    def _get(self, lib: str, name: str, argtypes):
+        key = (lib, name)
+        fn = self._fn.get(key)
+        if fn is None:
+            fn = getattr(build.load_library(lib), name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+            self._fn[key] = fn
+        return fn
+
+    def _run(self, lib: str, name: str, argtypes, *args):
+        fn = self._get(lib, name, argtypes)
+        code = fn(*args, torch.cuda.current_stream().cuda_stream)
+        if code != 0:
+            msg = build.load_library(lib).lle_error_string(code).decode()
+            raise KernelError(f"{name} failed to launch: {msg} (hip error {code})")
+
+    # -- embedding -----------------------------------------------------------
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+        """ids int32 [N], table [V, H] -> float32 [N, H] (the residual stream)."""
+        _dev(ids, "ids", torch.int32)
+        _dev(table, "embedding table")
+        _need(ids.dim() == 1 and table.dim() == 2, "embedding wants ids [N] and a table [V, H]")
+        N, H = ids.shape[0], table.shape[1]
+        out = torch.empty((N, H), dtype=torch.float32, device=table.device)
+        self._run("elementwise", "lle_embedding", [_P, _P, _P, _I, _I, _I, _P],
+                  _ptr(ids), _ptr(table), _ptr(out), N, H, dtype_code(table.dtype))
+        return out
+
+    # -- norms ---------------------------------------------------------------
+    def add_rmsnorm(self, hidden, delta, weight, eps: float, out_dtype, rows=None) -> torch.Tensor:
+        """hidden float32 [N, H] (+ delta [N, H] of out_dtype) -> norm * weight, out_dtype.
+        Without `rows` the sum is written back to `hidden` and every row is normed;
+        with `rows` (int32 [R]) only those rows are read and nothing is written back."""
+        _dev(hidden, "hidden", torch.float32)
+        _dev(weight, "norm weight")
+        N, H = hidden.shape
+        _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        if delta is not None:
+            _dev(delta, "delta", out_dtype)
+            _need(delta.shape == hidden.shape, "delta must have the shape of hidden")
+        if rows is not None:
+            _dev(rows, "rows", torch.int32)
+            R = rows.shape[0]
+        else:
+            R = N
+        out = torch.empty((R, H), dtype=out_dtype, device=hidden.device)
+        self._run("norm", "lle_add_rmsnorm", [_P, _P, _P, _P, _I, _P, _I, _I, _F, _I, _P],
+                  _ptr(hidden), _ptr(delta), _ptr(rows), _ptr(weight), dtype_code(weight.dtype), _ptr(out),
+                  R, H, float(eps), dtype_code(out_dtype))
+        return out
+
+    def rmsnorm(self, x, weight, eps: float) -> torch.Tensor:
+        """x [R, H] -> x * rsqrt(mean(x^2) + eps) * weight, same type."""
+        _dev(x, "x")
+        _dev(weight, "norm weight")
+        R, H = x.shape
+        _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        out = torch.empty_like(x)
+        self._run("norm", "lle_rmsnorm", [_P, _P, _I, _P, _I, _I, _F, _I, _P],
+                  _ptr(x), _ptr(weight), dtype_code(weight.dtype), _ptr(out), R, H, float(eps), dtype_code(x.dtype))
+        return out
+
+    # -- matrix products -------------------------------------------------------
+    def linear(self, x, weight, out_dtype=None) -> torch.Tensor:
+        """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
+        kernel (a true 32-bit product); bfloat16 operands with a bfloat16 result go
+        to the library product, with a float32 result to the 32-bit-accumulate kernel."""
+        _dev(x, "x")
+        _dev(weight, "weight", x.dtype)
+        M, K = x.shape
+        N = weight.shape[0]
+        _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
+        out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
+            return torch.mm(x, weight.t())
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
+                  _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
+        return out
+
+    # -- attention ---------------------------------------------------------------
+    def qk_norm_rope_write(self, qkv, positions, slots, q_weight, k_weight, inv_freq, rotary_dim: int,
+                           eps: float, kv_layer, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                           write_kv: bool = True) -> torch.Tensor:
+        """qkv [N, (nq + 2 nkv) d] -> q [N, nq, d] normed and rotated; K (normed, rotated)
+        and V go to the pages `kv_layer` [pages, 2, nkv, page_size, d] at `slots` [N]."""
+        _dev(qkv, "qkv")
+        _dev(positions, "positions", torch.int32)
+        _dev(slots, "slots", torch.int32)
+        _dev(kv_layer, "kv_layer", qkv.dtype)
+        nq, nkv, d = num_q_heads, num_kv_heads, head_dim
+        N = qkv.shape[0]
+        _need(qkv.shape == (N, (nq + 2 * nkv) * d), "qkv has the wrong width")
+        _need(positions.shape == (N,) and slots.shape == (N,), "positions and slots must be [N]")
+        _need(kv_layer.dim() == 5 and kv_layer.shape[1] == 2 and kv_layer.shape[2] == nkv
+              and kv_layer.shape[4] == d, "kv_layer must be [pages, 2, nkv, page_size, d]")
+        _need(0 <= rotary_dim <= d and rotary_dim % 2 == 0, "rotary_dim must be even and <= head_dim")
+        wd = F32
+        for w, name in ((q_weight, "q_norm weight"), (k_weight, "k_norm weight")):
+            if w is not None:
+                _dev(w, name)
+                _need(w.shape == (d,), f"{name} must be [{d}]")
+                wd = dtype_code(w.dtype)
+        if q_weight is not None and k_weight is not None:
+            _need(q_weight.dtype == k_weight.dtype, "q_norm and k_norm weights must share a type")
+        if rotary_dim > 0:
+            _dev(inv_freq, "inv_freq", torch.float32)
+            _need(inv_freq.shape == (rotary_dim // 2,), "inv_freq must be [rotary_dim / 2]")
+        page_size = kv_layer.shape[3]
+        q_out = torch.empty((N, nq, d), dtype=qkv.dtype, device=qkv.device)
+        self._run("rope_kv", "lle_qk_norm_rope_write",
+                  [_P, _P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _P],
+                  _ptr(qkv), _ptr(positions), _ptr(slots), _ptr(q_weight), _ptr(k_weight), wd,
+                  _ptr(inv_freq) if rotary_dim > 0 else None, rotary_dim, float(eps), _ptr(q_out), _ptr(kv_layer),
+                  N, nq, nkv, d, page_size, kv_layer.stride(0), 1 if write_kv else 0, dtype_code(qkv.dtype))
+        return q_out
+
+    def paged_attention(self, q, kv_layer, block_table, seq_slots, cu_tokens, kv_lens, token_seq,
+                        window: Optional[int], scale: float, max_q_len: int = 0, max_kv_len: int = 0) -> torch.Tensor:
+        """q [N, nq, d] against the pages -> [N, nq * d].  `max_q_len`/`max_kv_len`
+        are host-side bounds of this batch (hints for choosing a kernel)."""
+        _dev(q, "q")
+        _dev(kv_layer, "kv_layer", q.dtype)
+        for t, name in ((block_table, "block_table"), (seq_slots, "seq_slots"), (cu_tokens, "cu_tokens"),
+                        (kv_lens, "kv_lens"), (token_seq, "token_seq")):
+            _dev(t, name, torch.int32)
+        N, nq, d = q.shape
+        nkv, page_size = kv_layer.shape[2], kv_layer.shape[3]
+        _need(kv_layer.shape[4] == d and kv_layer.shape[1] == 2, "kv_layer must be [pages, 2, nkv, page_size, d]")
+        _need(nq % nkv == 0, "q heads must be a multiple of kv heads")
+        _need(d <= self.MAX_HEAD_DIM, f"head_dim {d} is larger than the attention kernels take ({self.MAX_HEAD_DIM})")
+        _need(token_seq.shape == (N,), "token_seq must be [N]")
+        S = seq_slots.shape[0]
+        _need(cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "cu_tokens [S + 1], kv_lens [S]")
+        _need(block_table.dim() == 2, "block_table must be [slots, pages]")
+        out = torch.empty((N, nq * d), dtype=q.dtype, device=q.device)
+        self._run("attention", "lle_paged_attention_generic",
+                  [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P],
+                  _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
+                  _ptr(token_seq), _ptr(out), N, nq, nkv, d, page_size, kv_layer.stride(0), block_table.shape[1],
+                  int(window) if window else 0, float(scale), dtype_code(q.dtype))
+        return out
+
+    # -- feed-forward --------------------------------------------------------------
+    def silu_mul(self, gate_up) -> torch.Tensor:
+        """gate_up [N, 2 I] (gate columns first) -> silu(gate) * up, [N, I]."""
+        _dev(gate_up, "gate_up")
+        N, two_i = gate_up.shape
+        _need(two_i % 2 == 0, "gate_up must have an even width")
+        out = torch.empty((N, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+        self._run("elementwise", "lle_silu_mul", [_P, _P, _I, _I, _I, _P],
+                  _ptr(gate_up), _ptr(out), N, two_i // 2, dtype_code(gate_up.dtype))
+        return out
+
+    # -- picking tokens --------------------------------------------------------------
+    def argmax(self, logits) -> torch.Tensor:
+        """float32 [R, V] -> int32 [R], first maximum wins."""
+        _dev(logits, "logits", torch.float32)
+        R, V = logits.shape
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        self._run("sampling", "lle_argmax_rows", [_P, _P, _I, _I, _P], _ptr(logits), _ptr(out), R, V)
+        return out
+
+    def sample(self, logits, temperature, uniform) -> torch.Tensor:
+        """float32 logits [R, V], temperature [R] (<= 0: greedy), uniform [R] in [0, 1) -> int32 [R]."""
+        _dev(logits, "logits", torch.float32)
+        _dev(temperature, "temperature", torch.float32)
+        _dev(uniform, "uniform", torch.float32)
+        R, V = logits.shape
+        _need(temperature.shape == (R,) and uniform.shape == (R,), "temperature and uniform must be [R]")
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        self._run("sampling", "lle_sample_rows", [_P, _P, _P, _P, _I, _I, _P],
+                  _ptr(logits), _ptr(temperature), _ptr(uniform), _ptr(out), R, V)
+        return out
+
+
+_default: Optional[HipOps] = None
+
+
+def default_ops() -> HipOps:
+    global _default
+    if _default is None:
+        _default = HipOps()
+    return _default

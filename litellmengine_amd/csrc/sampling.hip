@@ -1,0 +1,129 @@
+// Picking tokens from 32-bit logits rows: greedy (first maximum wins, as
+// argmax_each_row_kernel, src/ops/argmax.cu:181-241) and temperature sampling
+// (the reference parses --temperature and then only warns, src/main.cpp:175-178).
+#include "common.h"
+
+LLE_DEFINE_ERROR_STRING()
+
+#define SAMPLE_THREADS 1024
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_rows_kernel(const float* __restrict__ logits,
+                                                                     int32_t* __restrict__ out, int V) {
+    __shared__ float s_val[SAMPLE_THREADS / LLE_WAVE];
+    __shared__ int s_idx[SAMPLE_THREADS / LLE_WAVE];
+    const float* row = logits + (int64_t)blockIdx.x * V;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        const float v = row[i];
+        if (v > best || best_i == 0x7fffffff) {  // strided ascending: first maximum of this thread
+            best = v;
+            best_i = i;
+        }
+    }
+    // a NaN never wins a ">" comparison; ties go to the smaller index
+    for (int o = LLE_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, LLE_WAVE);
+        const int oi = __shfl_xor(best_i, o, LLE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) {
+            best = ov;
+            best_i = oi;
+        }
+    }
+    const int lane = threadIdx.x % LLE_WAVE, wave = threadIdx.x / LLE_WAVE;
+    if (lane == 0) {
+        s_val[wave] = best;
+        s_idx[wave] = best_i;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < SAMPLE_THREADS / LLE_WAVE; ++w)
+            if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
+                best = s_val[w];
+                best_i = s_idx[w];
+            }
+        out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+    }
+}
+
+extern "C" int lle_argmax_rows(const void* logits, void* out, int R, int V, hipStream_t stream) {
+    if (R <= 0) return 0;
+    argmax_rows_kernel<<<R, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (int32_t*)out, V);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// p_i = exp((x_i - max) / T); the pick is the first i whose running sum of p
+// exceeds u * sum(p).  Thread t owns the contiguous ids [t c, (t + 1) c), so the
+// running sum is taken in id order.  Rows with T <= 0 are picked greedily.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits,
+                                                                     const float* __restrict__ temperature,
+                                                                     const float* __restrict__ uniform,
+                                                                     int32_t* __restrict__ out, int V) {
+    __shared__ float red[16];
+    __shared__ float s_part[SAMPLE_THREADS];
+    __shared__ int s_pick;
+    const float* row = logits + (int64_t)blockIdx.x * V;
+    const float T = temperature[blockIdx.x];
+    const int t = threadIdx.x;
+    const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+    const int lo = min(V, t * chunk), hi = min(V, lo + chunk);
+
+    float mx = -INFINITY;
+    int mx_i = V;
+    for (int i = lo; i < hi; ++i)
+        if (row[i] > mx) {
+            mx = row[i];
+            mx_i = i;
+        }
+    const float big = block_max(mx, red);
+    if (T <= 0.f) {  // greedy: smallest index that reaches the maximum
+        if (t == 0) s_pick = V;
+        __syncthreads();
+        if (mx == big && mx_i < V) atomicMin(&s_pick, mx_i);
+        __syncthreads();
+        if (t == 0) out[blockIdx.x] = s_pick < V ? s_pick : 0;
+        return;
+    }
+    const float inv_t = 1.0f / T;
+    float part = 0.f;
+    for (int i = lo; i < hi; ++i) part += expf((row[i] - big) * inv_t);
+    s_part[t] = part;
+    __syncthreads();
+    if (t == 0) {
+        // sequential scan over 1024 partial sums: fixed order, once per row
+        float run = 0.f;
+        for (int k = 0; k < SAMPLE_THREADS; ++k) {
+            const float p = s_part[k];
+            s_part[k] = run;  // exclusive prefix
+            run += p;
+        }
+        red[0] = run;
+        s_pick = V;
+    }
+    __syncthreads();
+    const float total = red[0];
+    const float target = uniform[blockIdx.x] * total;
+    const float before = s_part[t];
+    if (lo < hi && target >= before && target < before + part) {
+        float run = before;
+        int pick = hi - 1;
+        for (int i = lo; i < hi; ++i) {
+            run += expf((row[i] - big) * inv_t);
+            if (run > target) {
+                pick = i;
+                break;
+            }
+        }
+        atomicMin(&s_pick, pick);
+    }
+    __syncthreads();
+    if (t == 0) out[blockIdx.x] = s_pick < V ? s_pick : V - 1;
+}
+
+extern "C" int lle_sample_rows(const void* logits, const void* temperature, const void* uniform, void* out, int R,
+                               int V, hipStream_t stream) {
+    if (R <= 0) return 0;
+    sample_rows_kernel<<<R, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (const float*)temperature,
+                                                          (const float*)uniform, (int32_t*)out, V);
+    LLE_RETURN_LAUNCH_STATUS();
+}

@@ -1,0 +1,14 @@
+from .attention import PagedAttention
+from .base import Block, BuildContext, FeedForward, KVCacheSpec, Mixer, Norm, Part, PositionEncoding, StateSpec
+from .block import PreNormBlock
+from .embedding import Embedding
+from .feed_forward import GatedMLP
+from .linear import Linear
+from .norm import RMSNorm
+from .position import NoPositionEncoding, RotaryHalfSplit
+
+__all__ = [
+    "Block", "BuildContext", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
+    "NoPositionEncoding", "Norm", "PagedAttention", "Part", "PositionEncoding", "PreNormBlock", "RMSNorm",
+    "RotaryHalfSplit", "StateSpec",
+]

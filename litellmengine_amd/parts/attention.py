@@ -1,0 +1,109 @@
+"""Grouped-query attention over the paged cache.
+
+q/k/v projections (no bias) -> RMSNorm of each q and k head over head_dim with
+one weight [head_dim] for all heads, before the position encoding; v untouched
+-> position encoding of q and k -> K (ready to dot) and V written to the pages
+-> attention of every token of the step through the block table -> output
+projection.  src/model/qwen3.cpp:375-377, :391-407, :443-449, :464-481,
+:498-557, :565-567.  scale = 1/sqrt(head_dim) (src/ops/attention.cu:201); kv
+head of q head h is h // (nq // nkv) (:196-199).  The q/k norm is optional and
+the position encoding is a part of its own, so the same mixer serves models
+without either; `window` limits a query to the last `window` keys (the
+reference has full attention only).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..weights.spec import INIT_NORM, TensorSpec
+from .base import BuildContext, KVCacheSpec, Mixer, PositionEncoding
+from .linear import Linear
+
+
+class PagedAttention(Mixer):
+    def __init__(
+        self,
+        prefix: str,
+        hidden_size: int,
+        num_q_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        position: PositionEncoding,
+        qk_norm_eps: Optional[float] = None,
+        window: Optional[int] = None,
+        scale: Optional[float] = None,
+    ):
+        if num_q_heads % num_kv_heads:
+            raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+        self.prefix = prefix
+        self.nq, self.nkv, self.d = num_q_heads, num_kv_heads, head_dim
+        self.position = position
+        self.qk_norm_eps = qk_norm_eps
+        self.window = window
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
+        self.qkv = Linear(
+            [prefix + "q_proj.weight", prefix + "k_proj.weight", prefix + "v_proj.weight"],
+            hidden_size,
+            [num_q_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
+        )
+        self.o = Linear([prefix + "o_proj.weight"], num_q_heads * head_dim, [hidden_size])
+        self.q_norm_w = None
+        self.k_norm_w = None
+
+    def cache_spec(self) -> KVCacheSpec:
+        return KVCacheSpec(self.nkv, self.d, self.window)
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs = {**self.qkv.tensor_specs(), **self.o.tensor_specs()}
+        if self.qk_norm_eps is not None:
+            specs[self.prefix + "q_norm.weight"] = TensorSpec((self.d,), INIT_NORM)
+            specs[self.prefix + "k_norm.weight"] = TensorSpec((self.d,), INIT_NORM)
+        return specs
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.qkv.bind(weights, ctx)
+        self.o.bind(weights, ctx)
+        self.position.bind(weights, ctx)
+        if self.qk_norm_eps is not None:
+            qw = weights[self.prefix + "q_norm.weight"]
+            kw = weights[self.prefix + "k_norm.weight"]
+            if qw.dtype != kw.dtype:
+                qw, kw = qw.float(), kw.float()
+            self.q_norm_w, self.k_norm_w = qw.contiguous(), kw.contiguous()
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        ops = self.ctx.ops
+        qkv = self.qkv.forward(x)
+        fused = self.position.fused_rotary()
+        eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
+        group = cache.group
+        if fused is not None:
+            inv_freq, rot = fused
+            q = ops.qk_norm_rope_write(
+                qkv, step.positions, group.slot_mapping, self.q_norm_w, self.k_norm_w, inv_freq, rot, eps,
+                cache.kv, self.nq, self.nkv, self.d, cache.writes,
+            )
+        else:
+            # an encoding the fused kernel does not know: norm, encode, then write
+            N = qkv.shape[0]
+            qw, kw = self.nq * self.d, self.nkv * self.d
+            q = qkv[:, :qw].reshape(N * self.nq, self.d).contiguous()
+            k = qkv[:, qw : qw + kw].reshape(N * self.nkv, self.d).contiguous()
+            if self.qk_norm_eps is not None:
+                q = ops.rmsnorm(q, self.q_norm_w, eps)
+                k = ops.rmsnorm(k, self.k_norm_w, eps)
+            q, k = self.position.apply(q.view(N, self.nq, self.d), k.view(N, self.nkv, self.d), step.positions)
+            packed = torch.cat([q.reshape(N, qw), k.reshape(N, kw), qkv[:, qw + kw :]], dim=1).contiguous()
+            q = ops.qk_norm_rope_write(
+                packed, step.positions, group.slot_mapping, None, None, None, 0, 0.0,
+                cache.kv, self.nq, self.nkv, self.d, cache.writes,
+            )
+        a = ops.paged_attention(
+            q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens, step.token_seq,
+            self.window, self.scale, step.max_q_len, step.max_kv_len,
+        )
+        return self.o.forward(a)

@@ -1,0 +1,117 @@
+"""Interfaces of the parts a model is put together from.
+
+A part knows its own sizes and constants (given as parameters when it is made)
+and the names of its tensors; it never knows which model it sits in.  Parts are
+made without touching memory; `bind` hands them their tensors, and `forward`
+runs them on the flat token batch of one step.
+
+To add a part of some kind, subclass the matching interface below and use it
+from an architecture's builder; nothing else in the package refers to the
+concrete classes.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+
+from ..weights.spec import TensorSpec
+
+
+@dataclasses.dataclass
+class BuildContext:
+    """Where and how a model is materialised."""
+
+    dtype: torch.dtype  # activation/weight type: torch.bfloat16 or torch.float32
+    device: torch.device
+    ops: Any  # the kernel operations (csrc.ops.HipOps)
+
+
+@dataclasses.dataclass(frozen=True)
+class KVCacheSpec:
+    """Per-token cache need of a mixer: keys and values of `num_kv_heads` heads of
+    `head_dim`; with a `window` only the last `window` positions stay needed."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size per-request state of a mixer (zeroed when a request is admitted)."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        """Checkpoint tensors of this part, by full name."""
+        return {}
+
+    def bind(self, weights: Dict[str, torch.Tensor], ctx: BuildContext) -> None:
+        """Take the tensors named by `tensor_specs` out of `weights`."""
+        self.ctx = ctx
+
+
+class Norm(Part):
+    """forward(hidden, delta) adds `delta` (or nothing) into the 32-bit residual
+    stream `hidden` in place and returns the normed rows in the activation type;
+    with `rows` only those rows are read and `hidden` is left alone."""
+
+    def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], rows=None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into q and k.  `fused_rotary()` may return
+    (inv_freq float32 [rotary_dim / 2], rotary_dim) when the encoding is a
+    half-split rotation that the fused q/k kernel can apply itself; otherwise
+    `apply` is called on q [N, nq, d] and k [N, nkv, d] (it may work in place)."""
+
+    def fused_rotary(self):
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a request.
+
+    forward(x [N, hidden], step, cache) -> [N, hidden].  `step` is the
+    engine.batch.StepState of this step; `cache` is the cache.manager.LayerCache
+    of the plan entry being run (pages of its group, the state rows, and whether
+    this entry writes)."""
+
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(x [N, hidden]) -> [N, hidden], token by token."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norm, mixer and feed-forward around the residual stream.
+
+    forward(hidden, delta, step, cache) -> delta': `hidden` is the 32-bit
+    residual stream [N, hidden]; `delta` is what the previous block still has to
+    add to it (None for the first); the return value is what this block leaves
+    to be added by whoever comes next."""
+
+    mixer: Mixer
+
+    def forward(self, hidden, delta, step, cache):
+        raise NotImplementedError

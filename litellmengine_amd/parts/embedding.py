@@ -1,0 +1,28 @@
+"""Token embedding: h[t, :] = E[ids[t], :] (src/layers/embedding.cu:75-87); the
+rows leave as float32, the type of the residual stream."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..weights.spec import INIT_NORMAL, TensorSpec
+from .base import BuildContext, Part
+
+
+class Embedding(Part):
+    def __init__(self, name: str, vocab_size: int, hidden_size: int):
+        self.name = name
+        self.vocab_size = vocab_size
+        self.hidden_size = hidden_size
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.name: TensorSpec((self.vocab_size, self.hidden_size), INIT_NORMAL)}
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.weight = weights[self.name].to(ctx.dtype).contiguous()
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        return self.ctx.ops.embedding(ids, self.weight)

@@ -1,0 +1,29 @@
+"""RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w; the weight multiplies directly,
+no bias, no mean subtraction (src/layers/rms_norm.cu:81-93).  The residual add
+that precedes a norm in the block is folded into the same kernel."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..weights.spec import INIT_NORM, TensorSpec
+from .base import BuildContext, Norm
+
+
+class RMSNorm(Norm):
+    def __init__(self, name: str, size: int, eps: float):
+        self.name = name
+        self.size = size
+        self.eps = float(eps)
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {self.name: TensorSpec((self.size,), INIT_NORM)}
+
+    def bind(self, weights, ctx: BuildContext) -> None:
+        self.ctx = ctx
+        self.weight = weights[self.name].contiguous()  # bfloat16 or float32, as stored
+
+    def forward(self, hidden, delta, rows=None) -> torch.Tensor:
+        return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)

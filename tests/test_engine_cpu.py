@@ -1,0 +1,47 @@
+"""The cache, the batch layout and the step function, exercised on the CPU with
+plain torch forms of the kernels (tests/torch_ops.py) in place of the HIP ones,
+against the plain whole-sequence implementation."""
+import pytest
+import torch
+
+from litellmengine_amd.cache import CacheManager
+from litellmengine_amd.engine import ModelRunner, StepEntry
+from litellmengine_amd.models import load_model
+from tests.plain import qwen3_plain as plain
+from tests.tiny import CONFIGS, PAGE_SIZES, make_model_dir, random_tokens
+from tests.torch_ops import TorchOps
+
+
+def make_runner(model_dir, page_size, num_pages, max_requests=4, dtype=torch.float32):
+    model = load_model(model_dir, dtype, device="cpu", ops=TorchOps())
+    cache = CacheManager(model, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                         dtype=dtype, device="cpu")
+    return ModelRunner(model, cache)
+
+
+def run_cut(runner, tokens, cuts):
+    """Feed `tokens` in portions of the sizes in `cuts`; logits of every position."""
+    slot = runner.admit()
+    rows = []
+    at = 0
+    for c in cuts:
+        part = tokens[at : at + c]
+        rows.append(runner.step([StepEntry(slot, part, list(range(len(part))))]))
+        at += c
+    assert at == len(tokens)
+    runner.release(slot)
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_cuts_match_plain(tmp_path, which):
+    d = make_model_dir(tmp_path, which)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(45, cfg["vocab_size"], 7)
+    want = plain.model_logits_fast(tokens, w, cfg)
+    runner = make_runner(d, PAGE_SIZES[which], 16)
+    for cuts in ([45], [13] + [1] * 32, [2, 7, 16, 3, 2, 15], [1] * 45):
+        got = run_cut(runner, tokens, cuts)
+        err = (got.double() - want).abs().max().item()
+        assert err < 2e-5, (cuts, err)
+    assert all(g.pool.num_held == 0 for g in runner.cache.groups)

@@ -1,0 +1,44 @@
+"""Tiny Qwen3 configurations for the tests.  Between them every size and option
+differs: layers, width, head counts and group size, head size (q width equal to
+the width or not), feed-forward width, vocabulary (a power of two or odd),
+rotary base, eps, tied or untied head, all-keys layers or layers with a window."""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from litellmengine_amd.config import Qwen3Config
+from litellmengine_amd.weights import write_model_dir
+
+TINY_A = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=2, hidden_size=64,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128, vocab_size=256,
+    rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+)
+TINY_B = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=3, hidden_size=96,
+    num_attention_heads=8, num_key_value_heads=2, head_dim=32, intermediate_size=200, vocab_size=503,
+    rope_theta=1000000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+)
+# layers with a window beside layers that see everything: two cache groups
+TINY_C = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=4, hidden_size=80,
+    num_attention_heads=6, num_key_value_heads=3, head_dim=48, intermediate_size=136, vocab_size=311,
+    rope_theta=500000.0, rms_norm_eps=3e-6, tie_word_embeddings=False, sliding_window=20,
+    layer_types=["sliding_attention", "full_attention", "sliding_attention", "sliding_attention"],
+)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+PAGE_SIZES = {"A": 4, "B": 8, "C": 16}
+
+
+def make_model_dir(tmp_path, which: str, seed: int = 1234, dtype=torch.float32) -> str:
+    cfg = Qwen3Config.from_dict(CONFIGS[which])
+    path = os.path.join(str(tmp_path), f"tiny_{which}_{seed}")
+    write_model_dir(cfg, path, seed, dtype)
+    return path
+
+
+def random_tokens(n: int, vocab: int, seed: int):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
