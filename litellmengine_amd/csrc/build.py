@@ -75,14 +75,23 @@ def _writable_dir(path: str) -> bool:
         return False
 
 
+_lib_dir = None
+_lib_dir_lock = threading.Lock()
+
+
 def lib_dir() -> str:
-    in_tree = os.path.join(_HERE, "lib")
-    if _writable_dir(in_tree):
-        return in_tree
-    fallback = os.path.join(tempfile.gettempdir(), f"litellmengine_amd-{os.getuid()}", "lib")
-    if _writable_dir(fallback):
-        return fallback
-    raise BuildError(f"neither {in_tree} nor {fallback} can be written")
+    global _lib_dir
+    with _lib_dir_lock:
+        if _lib_dir is None:
+            in_tree = os.path.join(_HERE, "lib")
+            fallback = os.path.join(tempfile.gettempdir(), f"litellmengine_amd-{os.getuid()}", "lib")
+            if _writable_dir(in_tree):
+                _lib_dir = in_tree
+            elif _writable_dir(fallback):
+                _lib_dir = fallback
+            else:
+                raise BuildError(f"neither {in_tree} nor {fallback} can be written")
+        return _lib_dir
 
 
 def _source_hash(name: str) -> str:

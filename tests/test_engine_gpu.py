@@ -1,0 +1,47 @@
+"""The engine on the GPU against the plain implementation: whole prompts, the
+last tokens one by one, portions of changing size; float32 and bfloat16."""
+import pytest
+import torch
+
+from litellmengine_amd.cache import CacheManager
+from litellmengine_amd.engine import ModelRunner, StepEntry
+from litellmengine_amd.models import load_model
+from tests.plain import qwen3_plain as plain
+from tests.tiny import PAGE_SIZES, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+
+
+def make_runner(model_dir, dtype, page_size, num_pages, max_requests=4):
+    model = load_model(model_dir, dtype)
+    cache = CacheManager(model, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                         dtype=model.ctx.dtype, device=model.ctx.device)
+    return ModelRunner(model, cache)
+
+
+def run_cut(runner, tokens, cuts):
+    slot = runner.admit()
+    rows, at = [], 0
+    for c in cuts:
+        part = tokens[at : at + c]
+        rows.append(runner.step([StepEntry(slot, part, list(range(len(part))))]).cpu())
+        at += c
+    runner.release(slot)
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_cuts_match_plain(tmp_path, which, dtype):
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(77, cfg["vocab_size"], 7)
+    want = plain.model_logits_fast(tokens, w, cfg)
+    runner = make_runner(d, dtype, PAGE_SIZES[which], 80 // PAGE_SIZES[which] + 1)
+    for cuts in ([77], [45] + [1] * 32, [2, 7, 16, 3, 2, 15, 30, 2]):
+        got = run_cut(runner, tokens, cuts)
+        err = (got.double() - want).abs().max().item()
+        assert err < TOL[dtype], (cuts, err)
+    assert all(g.pool.num_held == 0 for g in runner.cache.groups)

@@ -1,0 +1,254 @@
+"""Each HIP kernel alone against its plain torch form (tests/torch_ops.py), in
+float32 and bfloat16, at sizes other than the tiny models': widths and
+vocabularies that are no power of two, head sizes in steps of 16, odd page sizes."""
+import math
+
+import pytest
+import torch
+
+from tests.torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+REF = TorchOps(torch.float64)
+
+
+def ops():
+    from litellmengine_amd.csrc.ops import default_ops
+
+    return default_ops()
+
+
+def tol(dtype, scale=1.0):
+    return (2e-5 if dtype == torch.float32 else 2e-2) * scale
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [48, 1000, 4096])
+def test_embedding(dtype, H):
+    table = rnd((333, H), dtype, 1)
+    ids = torch.tensor([0, 332, 5, 5, 17], dtype=torch.int32).cuda()
+    got = ops().embedding(ids, table)
+    assert got.dtype == torch.float32
+    assert torch.equal(got, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,wdtype", [(80, None), (1000, torch.float32), (5120, None), (9000, None)])
+def test_add_rmsnorm(dtype, H, wdtype):
+    N = 7
+    hidden = rnd((N, H), torch.float32, 2, 3.0)
+    delta = rnd((N, H), dtype, 3)
+    w = (1 + 0.1 * rnd((H,), torch.float32, 4)).to(wdtype or dtype)
+    h_ref = hidden.clone()
+    want = REF.add_rmsnorm(h_ref, delta, w, 1e-5, dtype)
+    got = ops().add_rmsnorm(hidden, delta, w, 1e-5, dtype)
+    assert torch.allclose(hidden, h_ref, atol=1e-6), "the residual sum is written back"
+    assert (got.double() - want.double()).abs().max() < tol(dtype, 4)
+    # no delta: hidden unchanged
+    before = hidden.clone()
+    got = ops().add_rmsnorm(hidden, None, w, 1e-5, dtype)
+    assert torch.equal(hidden, before)
+    assert (got.double() - REF.add_rmsnorm(before.clone(), None, w, 1e-5, dtype).double()).abs().max() < tol(dtype, 4)
+    # row list: only those rows, nothing written back
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32).cuda()
+    got = ops().add_rmsnorm(hidden, delta, w, 1e-5, dtype, rows=rows)
+    assert torch.equal(hidden, before)
+    want = REF.add_rmsnorm(before.clone(), delta, w, 1e-5, dtype, rows=rows)
+    assert got.shape == (3, H)
+    assert (got.double() - want.double()).abs().max() < tol(dtype, 4)
+
+
+def test_rmsnorm_reference_vector():
+    # input and weight of tests/test_rms_norm.cpp:57-64; expected by hand:
+    # row 0: mean(x^2) = 7.5, row 1: mean(x^2) = 6
+    x = torch.tensor([[1.0, 2, 3, 4], [2, 0, -2, 4]]).cuda()
+    w = torch.tensor([1.0, 1.5, 2.0, 0.5]).cuda()
+    got = ops().rmsnorm(x, w, 1e-6).cpu()
+    r0, r1 = 1 / math.sqrt(7.5 + 1e-6), 1 / math.sqrt(6 + 1e-6)
+    want = torch.tensor([[1 * r0, 3 * r0, 6 * r0, 2 * r0], [2 * r1, 0, -4 * r1, 2 * r1]])
+    assert torch.allclose(got, want, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("I", [8, 200, 12288])
+def test_silu_mul(dtype, I):
+    gu = rnd((5, 2 * I), dtype, 5, 2.0)
+    got = ops().silu_mul(gu)
+    want = REF.silu_mul(gu)
+    assert (got.double() - want.double()).abs().max() < tol(dtype, 4)
+
+
+def test_silu_mul_reference_vector():
+    # tests/test_silu_and_mul.cpp:48-56
+    g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])
+    u = torch.tensor([[1.0, 2, -1, 0.5], [3, -2, 4, -3]])
+    got = ops().silu_mul(torch.cat([g, u], dim=1).cuda()).cpu()
+    want = torch.nn.functional.silu(g) * u
+    assert torch.allclose(got, want, atol=1e-6)
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
+                                                (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("M,N,K", [(1, 503, 96), (2, 4, 3), (5, 130, 70), (67, 257, 200), (33, 1000, 4096)])
+def test_linear(in_dtype, out_dtype, M, N, K):
+    x = rnd((M, K), in_dtype, 6)
+    w = rnd((N, K), in_dtype, 7, 0.05)
+    got = ops().linear(x, w, out_dtype)
+    want = x.double() @ w.double().t()
+    assert got.dtype == out_dtype
+    lim = 1e-5 if out_dtype == torch.float32 and in_dtype == torch.float32 else (2e-5 if out_dtype == torch.float32 else 2e-2)
+    assert (got.double() - want).abs().max() < lim * max(1.0, want.abs().max().item())
+
+
+def test_linear_reference_vector():
+    # tests/test_linear.cpp:63-78: X 2x3, W 4x3
+    x = torch.tensor([[1.0, 2, 3], [4, 5, 6]]).cuda()
+    w = torch.tensor([[1.0, 2, 3], [4, 5, 6], [-1, 0, 1], [2, -3, 4]]).cuda()
+    want = torch.tensor([[14.0, 32, 2, 8], [32, 77, 2, 17]])
+    assert torch.equal(ops().linear(x, w).cpu(), want)
+
+
+def make_cache(num_pages, nkv, P, d, dtype, seed):
+    return rnd((num_pages, 2, nkv, P, d), dtype, seed)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,rot,norm", [(4, 2, 16, 4, 16, True), (6, 3, 48, 3, 48, True),
+                                                 (8, 1, 128, 16, 128, True), (2, 2, 80, 8, 32, False),
+                                                 (3, 1, 256, 5, 0, True)])
+def test_qk_norm_rope_write(dtype, nq, nkv, d, P, rot, norm):
+    N, pages = 9, 6
+    qkv = rnd((N, (nq + 2 * nkv) * d), dtype, 8)
+    positions = torch.tensor([0, 1, 2, 50, 51, 7, 1000, 3, 4], dtype=torch.int32).cuda()
+    slots = torch.tensor([0, 5, 9, -1, pages * P - 1, 2, 3, 11, 7], dtype=torch.int32).cuda()
+    qw = (1 + 0.1 * rnd((d,), torch.float32, 9)).to(dtype) if norm else None
+    kw = (1 + 0.1 * rnd((d,), torch.float32, 10)).to(dtype) if norm else None
+    inv = None
+    if rot:
+        i = torch.arange(rot // 2, dtype=torch.float64)
+        inv = (1e6 ** (-(2.0 * i) / rot)).float().cuda()
+    kv_got = make_cache(pages, nkv, P, d, dtype, 11)
+    kv_ref = kv_got.clone()
+    q_got = ops().qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv_got, nq, nkv, d)
+    q_ref = REF.qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv_ref, nq, nkv, d)
+    t = tol(dtype, 8)
+    assert (q_got.double() - q_ref.double()).abs().max() < t
+    assert (kv_got.double() - kv_ref.double()).abs().max() < t
+    # a reader entry leaves the pages alone
+    kv2 = kv_ref.clone()
+    ops().qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv2, nq, nkv, d, write_kv=False)
+    assert torch.equal(kv2, kv_ref)
+
+
+def test_rotary_reference_vector():
+    # q of tests/test_rotary.cpp:98-122: positions {0, 2}, d = 4, theta 1e4.
+    # position 0 is the identity; at position 2 pair (x[i], x[i+2]) turns by 2 * theta^(-2i/4)
+    q = torch.tensor([[1.0, 2, 3, 4, -1, 0.5, 2, -0.5], [0, 1, -2, 3, 4, -1, 0.25, -0.75]])
+    qkv = torch.cat([q, torch.zeros(2, 8)], dim=1).cuda()  # nq = 2, nkv = 1, d = 4
+    positions = torch.tensor([0, 2], dtype=torch.int32).cuda()
+    slots = torch.tensor([-1, -1], dtype=torch.int32).cuda()
+    inv = torch.tensor([1.0, 1e4 ** -0.5]).cuda()
+    kv = torch.zeros(1, 2, 1, 4, 4).cuda()
+    got = ops().qk_norm_rope_write(qkv, positions, slots, None, None, inv, 4, 0.0, kv, 2, 1, 4).cpu()
+    assert torch.allclose(got[0].reshape(-1), q[0], atol=1e-7)
+    x = q[1].reshape(2, 4)
+    want = torch.empty(2, 4)
+    for i, f in enumerate([1.0, 0.01]):
+        c, s = math.cos(2 * f), math.sin(2 * f)
+        want[:, i] = x[:, i] * c - x[:, i + 2] * s
+        want[:, i + 2] = x[:, i + 2] * c + x[:, i] * s
+    assert torch.allclose(got[1], want, atol=1e-6)
+
+
+def attention_case(dtype, nq, nkv, d, P, window, lens, seed=12, pages=40, max_pages=12):
+    """lens: list of (past, q_len).  Builds a cache with random pages in a
+    scrambled block table and random q."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(lens)
+    kv = make_cache(pages, nkv, P, d, dtype, seed + 1)
+    perm = torch.randperm(pages, generator=g).tolist()
+    table = torch.full((5, max_pages), -1, dtype=torch.int32)
+    slots = torch.randperm(5, generator=g)[:S].tolist()
+    cu, kv_lens, token_seq = [0], [], []
+    for s, (past, ql) in enumerate(lens):
+        n_pages = (past + ql + P - 1) // P
+        assert n_pages <= max_pages
+        for i in range(n_pages):
+            table[slots[s], i] = perm.pop()
+        cu.append(cu[-1] + ql)
+        kv_lens.append(past + ql)
+        token_seq += [s] * ql
+    N = cu[-1]
+    q = rnd((N, nq, d), dtype, seed + 2)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32).cuda()
+    args = (q, kv, table.cuda(), i32(slots), i32(cu), i32(kv_lens), i32(token_seq), window, 1.0 / math.sqrt(d))
+    return args, max(l for _, l in lens), max(kv_lens)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(4, 2, 16, 4, None), (6, 3, 48, 3, None), (8, 2, 128, 16, None),
+                                               (8, 8, 64, 16, 7), (5, 1, 80, 8, 20), (2, 1, 256, 16, None)])
+def test_paged_attention(dtype, nq, nkv, d, P, window):
+    lens = [(0, 9), (17, 1), (30, 2), (5, 11)]
+    args, mq, mk = attention_case(dtype, nq, nkv, d, P, window, lens)
+    got = ops().paged_attention(*args, mq, mk)
+    want = REF.paged_attention(*args)
+    assert (got.double() - want.double()).abs().max() < tol(dtype, 2)
+
+
+def test_attention_single_token_returns_value():
+    # tests/test_attention.cpp:220-281: one token sees only itself, out == V
+    args, mq, mk = attention_case(torch.float32, 4, 2, 16, 4, None, [(0, 1)])
+    got = ops().paged_attention(*args, mq, mk).reshape(1, 4, 16)
+    q, kv, table, slots = args[0], args[1], args[2], args[3]
+    page = int(table[int(slots[0]), 0])
+    v = kv[page, 1, :, 0, :]  # [nkv, d]
+    assert torch.allclose(got[0], v.repeat_interleave(2, dim=0), atol=1e-6)
+
+
+def test_attention_far_key_stands_out():
+    """One key far back is made to dominate: the output must be its value row."""
+    dtype, nq, nkv, d, P = torch.float32, 2, 1, 32, 16
+    args, mq, mk = attention_case(dtype, nq, nkv, d, P, None, [(299, 1)], pages=40, max_pages=20)
+    q, kv, table, slots = args[0], args[1], args[2], args[3]
+    far = 37
+    page, off = int(table[int(slots[0]), far // P]), far % P
+    kv[page, 0, 0, off, :] = q[0, 0] * 50.0
+    got = ops().paged_attention(*args, mq, mk).reshape(1, nq, d)
+    assert torch.allclose(got[0, 0], kv[page, 1, 0, off, :], atol=1e-4)
+
+
+@pytest.mark.parametrize("V", [7, 503, 151936])
+def test_argmax_and_sample(V):
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn((6, V), generator=g).cuda()
+    logits[1, V // 2] = 50.0
+    logits[2, 0] = 60.0
+    logits[3, V - 1] = 60.0
+    logits[4, :] = 1.0  # all equal: the first wins
+    logits[5, V - 1] = 9.0
+    logits[5, V // 3] = 9.0  # tie: the lower index wins
+    got = ops().argmax(logits).cpu().tolist()
+    want = torch.argmax(logits.cpu(), dim=-1).tolist()
+    assert got == want
+    assert got[4] == 0 and got[5] == V // 3
+    temperature = torch.tensor([0.7, 1.0, 0.0, 2.5, 1.0, 0.3]).cuda()
+    for seed in range(4):
+        u = torch.rand((6,), generator=torch.Generator().manual_seed(seed)).cuda()
+        got = ops().sample(logits, temperature, u).cpu().tolist()
+        want = REF.sample(logits.cpu(), temperature.cpu(), u.cpu()).tolist()
+        for r in range(6):
+            if got[r] != want[r]:
+                # rounding may move a pick across a boundary of the running sum by one id
+                p = torch.softmax(logits[r].double().cpu() / max(float(temperature[r]), 1e-9), 0)
+                cdf = torch.cumsum(p, 0)
+                lo, hi = sorted((got[r], want[r]))
+                assert abs(float(cdf[hi - 1]) - float(u[r])) < 1e-4 and hi - lo <= 2, (r, got[r], want[r])
+    assert ops().sample(logits, temperature, u).cpu().tolist()[2] == 0
