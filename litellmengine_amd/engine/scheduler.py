@@ -1,0 +1,165 @@
+"""The scheduler: which tokens of which requests run in the next step.
+
+The reference has no scheduler object: callers prefill every request alone and
+whole, then loop `decode_batch` over the unfinished ones, with a pool sized for
+the worst case so that pages never run out
+(src/benchmark/generation_benchmark.cpp:259-315); a shortage throws from
+`ensure_blocks` up to `main` (src/engine/block_table_manager.cpp:82-84).
+
+Here, every step:
+ 1. requests that are decoding (one pending token) come first, then requests
+    with prompt tokens left, oldest first; each gets min(pending, prefill_chunk,
+    what is left of max_tokens_per_step) tokens;
+ 2. if the pages for that are not there, the YOUNGEST running request is
+    preempted: its pages and slot are given back, its cache is forgotten
+    (cached_len = 0) and it waits at the FRONT of the queue to be recomputed
+    (prompt and what it generated so far); repeated until the step fits.  No
+    request is admitted in a step that preempted;
+ 3. otherwise waiting requests are admitted in order while a slot, budget and
+    the pages for their first portion are there.
+A request that could never fit (its last cached position needs more pages than
+a group has, or than a request may hold) is refused when it is added.  Finished
+requests give their pages back at once.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+from typing import Deque, Dict, List, Optional, Sequence
+
+from ..cache import CacheManager, OutOfPages
+from .request import Request, RequestStatus
+
+
+@dataclasses.dataclass(frozen=True)
+class Portion:
+    """`num_tokens` tokens of `request` from its `cached_len` on; `samples` when
+    the portion reaches the end of what the request has, so a token is drawn."""
+
+    request: Request
+    start: int
+    num_tokens: int
+    samples: bool
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_tokens_per_step: int = 2048, prefill_chunk: Optional[int] = None):
+        if max_tokens_per_step <= 0:
+            raise ValueError("max_tokens_per_step must be positive")
+        if prefill_chunk is not None and prefill_chunk <= 0:
+            raise ValueError("prefill_chunk must be positive")
+        self.cache = cache
+        self.max_tokens_per_step = max_tokens_per_step
+        self.prefill_chunk = prefill_chunk or max_tokens_per_step
+        self.waiting: Deque[Request] = collections.deque()
+        self.running: List[Request] = []
+        self.requests: Dict[int, Request] = {}
+        self._next_id = 0
+        self._admissions = 0
+        self.num_preemptions = 0
+
+    # -- adding ---------------------------------------------------------------------
+    def add_request(self, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_id: int = -1,
+                    temperature: float = 0.0, seed: int = 0) -> Request:
+        """src/engine/paged_generate_engine.cpp:57-79: a prompt must not be empty,
+        max_new_tokens >= 0; 0 finishes at once."""
+        if len(prompt_ids) == 0:
+            raise ValueError("a request needs a non-empty prompt")
+        if max_new_tokens < 0:
+            raise ValueError("max_new_tokens must be >= 0")
+        if temperature < 0:
+            raise ValueError("temperature must be >= 0")
+        req = Request(self._next_id, [int(t) for t in prompt_ids], len(prompt_ids), max_new_tokens,
+                      int(eos_token_id), float(temperature), int(seed))
+        self._next_id += 1
+        self.requests[req.request_id] = req
+        if max_new_tokens == 0:
+            req.status = RequestStatus.FINISHED
+            return req
+        longest = req.prompt_len + max_new_tokens - 1  # the last token drawn is never cached
+        for group in self.cache.groups:
+            pages = group.pages_for(longest)
+            if group.window is None and pages > group.pool.num_pages:
+                raise ValueError(
+                    f"request of {req.prompt_len} prompt + {max_new_tokens} new tokens needs {pages} pages, "
+                    f"the cache has {group.pool.num_pages}"
+                )
+            if pages > group.max_pages_per_request:
+                raise ValueError(
+                    f"request needs {pages} pages, a request may hold {group.max_pages_per_request}"
+                )
+        self.waiting.append(req)
+        return req
+
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # -- one step ---------------------------------------------------------------------
+    def schedule(self) -> List[Portion]:
+        budget = self.max_tokens_per_step
+        order = [r for r in self.running if r.extend_len == 1] + [r for r in self.running if r.extend_len > 1]
+        plan: List[Portion] = []
+        for r in order:
+            if budget == 0:
+                break
+            n = min(r.extend_len, self.prefill_chunk, budget)
+            plan.append(Portion(r, r.cached_len, n, n == r.extend_len))
+            budget -= n
+
+        preempted = False
+        while plan and not self.cache.can_extend([(p.request.slot, p.start + p.num_tokens) for p in plan]):
+            if len(self.running) == 1:
+                raise OutOfPages("the only running request does not fit into the cache")
+            victim = max(self.running, key=lambda r: r.admitted_at)
+            self._preempt(victim)
+            preempted = True
+            budget += sum(p.num_tokens for p in plan if p.request is victim)
+            plan = [p for p in plan if p.request is not victim]
+
+        while not preempted and self.waiting and budget > 0 and self.cache.num_free_slots > 0:
+            r = self.waiting[0]
+            n = min(r.extend_len, self.prefill_chunk, budget)
+            slot = self.cache.admit()
+            wants = [(p.request.slot, p.start + p.num_tokens) for p in plan] + [(slot, n)]
+            if not self.cache.can_extend(wants):
+                self.cache.release(slot)
+                if not self.running:
+                    raise OutOfPages("the first waiting request does not fit into the empty cache")
+                break
+            self.waiting.popleft()
+            r.slot = slot
+            r.status = RequestStatus.RUNNING
+            r.admitted_at = self._admissions
+            self._admissions += 1
+            self.running.append(r)
+            plan.append(Portion(r, 0, n, n == r.extend_len))
+            budget -= n
+        return plan
+
+    def _preempt(self, r: Request) -> None:
+        self.cache.release(r.slot)
+        r.slot = -1
+        r.cached_len = 0
+        r.status = RequestStatus.WAITING
+        r.preemptions += 1
+        self.num_preemptions += 1
+        self.running.remove(r)
+        self.waiting.appendleft(r)
+
+    def update(self, plan: Sequence[Portion], sampled: Sequence[int]) -> List[Request]:
+        """After the step ran: advance the caches' lengths, append the drawn tokens
+        (one per portion with `samples`, in plan order), finish and free.
+        Returns the requests that finished in this step."""
+        done: List[Request] = []
+        it = iter(sampled)
+        for p in plan:
+            r = p.request
+            r.mark_forward_done(p.num_tokens)
+            if p.samples:
+                r.append_token(next(it))
+                if r.finished:
+                    self.cache.release(r.slot)
+                    r.slot = -1
+                    self.running.remove(r)
+                    done.append(r)
+        return done

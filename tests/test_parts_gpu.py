@@ -1,0 +1,270 @@
+"""Each model part alone against the plain implementation, and a toy
+architecture defined HERE (a mixer with state of its own, another position
+encoding, a block that runs twice, a layer that reads another layer's cache)
+that is registered, built and stepped without any change to the package."""
+import dataclasses
+import math
+
+import pytest
+import torch
+
+from litellmengine_amd.cache import CacheManager
+from litellmengine_amd.config import register_architecture
+from litellmengine_amd.engine import ModelRunner, StepEntry
+from litellmengine_amd.models import DecoderLM, PlanEntry, make_context, random_model
+from litellmengine_amd.parts import (Embedding, GatedMLP, Linear, Mixer, PagedAttention, PositionEncoding,
+                                     PreNormBlock, RMSNorm, RotaryHalfSplit, StateSpec)
+from litellmengine_amd.weights import TensorSpec, random_weights
+from tests.plain import qwen3_plain as plain
+from tests.tiny import random_tokens
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+TOL = {torch.float32: 3e-5, torch.bfloat16: 4e-2}
+
+
+def bound(part, dtype, seed=0):
+    """Give `part` seeded random weights (rounded to bfloat16 so that both types see
+    the same values); returns (context, weights as float64 on the CPU)."""
+    ctx = make_context(dtype)
+    w = random_weights(part.tensor_specs(), seed, torch.bfloat16, "cpu", include_optional=True)
+    part.bind({k: v.to(ctx.device) for k, v in w.items()}, ctx)
+    return ctx, {k: v.to(D) for k, v in w.items()}
+
+
+def x_of(shape, dtype, seed, scale=1.0):
+    x = (torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale).to(torch.bfloat16)
+    return x.to(dtype).cuda(), x.to(D)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_norm_embedding_mlp(dtype):
+    lin = Linear(["a.weight", "b.weight"], 72, [40, 24])
+    ctx, w = bound(lin, dtype)
+    x, xp = x_of((5, 72), dtype, 1)
+    want = torch.cat([plain.linear(xp, w["a.weight"]), plain.linear(xp, w["b.weight"])], dim=1)
+    assert (lin.forward(x).cpu().double() - want).abs().max() < TOL[dtype]
+
+    norm = RMSNorm("n.weight", 72, 1e-5)
+    ctx, w = bound(norm, dtype)
+    hidden = torch.randn(5, 72).cuda()
+    delta, dp = x_of((5, 72), dtype, 2)
+    want_h = hidden.cpu().double() + dp
+    got = norm.forward(hidden, delta)
+    assert (hidden.cpu().double() - want_h).abs().max() < 1e-6
+    assert (got.cpu().double() - plain.rms_norm(want_h, w["n.weight"], 1e-5)).abs().max() < TOL[dtype] * 4
+
+    emb = Embedding("e.weight", 101, 56)
+    ctx, w = bound(emb, dtype)
+    ids = torch.tensor([0, 100, 7], dtype=torch.int32).cuda()
+    assert torch.equal(emb.forward(ids).cpu().double(), plain.embedding([0, 100, 7], w["e.weight"]))
+
+    mlp = GatedMLP("m.", 72, 136)
+    ctx, w = bound(mlp, dtype)
+    x, xp = x_of((6, 72), dtype, 3, 3.0)
+    want = plain.gated_mlp(xp, w["m.gate_proj.weight"], w["m.up_proj.weight"], w["m.down_proj.weight"])
+    assert (mlp.forward(x).cpu().double() - want).abs().max() < TOL[dtype]
+
+
+def one_block_model(block, hidden, vocab=50):
+    return DecoderLM(None, Embedding("e.weight", vocab, hidden), [block], [PlanEntry(0)],
+                     RMSNorm("fn.weight", hidden, 1e-6), Linear(["head.weight"], hidden, [vocab]), tied_head=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_mixer_and_block_alone(dtype, window):
+    """The attention mixer inside one pre-norm block, stepped in two portions and
+    then one token, against plain.decoder_layer on the whole sequence."""
+    H, nq, nkv, d, I = 72, 6, 2, 16, 100
+    p = "model.layers.0."
+    block = PreNormBlock(
+        RMSNorm(p + "input_layernorm.weight", H, 1e-5),
+        PagedAttention(p + "self_attn.", H, nq, nkv, d, RotaryHalfSplit(d, 5e4), qk_norm_eps=1e-5, window=window),
+        RMSNorm(p + "post_attention_layernorm.weight", H, 1e-5),
+        GatedMLP(p + "mlp.", H, I),
+    )
+    model = one_block_model(block, H)
+    ctx, w = bound(model, dtype)
+    model.ctx = ctx
+    cache = CacheManager(model, page_size=4, num_pages=8, max_requests=2, dtype=dtype, device=ctx.device)
+    runner = ModelRunner(model, cache)
+    T = 19
+    ids = random_tokens(T, 50, 4)
+    cfg = dict(num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, rms_norm_eps=1e-5, rope_theta=5e4)
+    h = plain.decoder_layer(plain.embedding(ids, w["e.weight"]), list(range(T)), w, 0, cfg, window)
+    want = plain.fast_linear(plain.rms_norm(h, w["fn.weight"], 1e-6), w["head.weight"])
+    slot = runner.admit()
+    got = torch.cat([runner.step([StepEntry(slot, ids[a:b], list(range(b - a)))]).cpu() for a, b in ((0, 11), (11, 18), (18, 19))])
+    assert (got.double() - want).abs().max() < TOL[dtype]
+
+
+# ---------------------------------------------------------------------------------------
+# a toy architecture, defined in this test only
+# ---------------------------------------------------------------------------------------
+class RunningMeanMixer(Mixer):
+    """y_t = W mean(x_0 .. x_t): needs no keys or values, only a running sum and a
+    count per request — fixed-size state that the cache manager carries."""
+
+    def __init__(self, name, hidden):
+        self.name, self.hidden = name, hidden
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.hidden, self.hidden))}
+
+    def state_spec(self):
+        return StateSpec((self.hidden + 1,), torch.float32)
+
+    def bind(self, weights, ctx):
+        self.ctx = ctx
+        self.weight = weights[self.name].to(ctx.dtype).contiguous()
+
+    def forward(self, x, step, cache):
+        out = torch.empty_like(x)
+        for q in step.seqs:
+            rows = slice(q.q_start, q.q_start + q.q_len)
+            state = cache.state[q.slot]
+            sums = state[:-1] + torch.cumsum(x[rows].float(), dim=0)
+            counts = state[-1] + torch.arange(1, q.q_len + 1, device=x.device, dtype=torch.float32)
+            out[rows] = (sums / counts[:, None]).to(x.dtype)
+            state[:-1] = sums[-1]
+            state[-1] = counts[-1]
+        return self.ctx.ops.linear(out, self.weight)
+
+
+class LearnedAdditivePosition(PositionEncoding):
+    """q += table[pos], k += table[pos]: not a rotation, so the mixer takes the
+    unfused path (norm, `apply`, then the page write)."""
+
+    def __init__(self, name, max_positions, head_dim):
+        self.name, self.max_positions, self.head_dim = name, max_positions, head_dim
+
+    def tensor_specs(self):
+        return {self.name: TensorSpec((self.max_positions, self.head_dim))}
+
+    def bind(self, weights, ctx):
+        self.ctx = ctx
+        self.table = weights[self.name].to(ctx.dtype).contiguous()
+
+    def apply(self, q, k, positions):
+        t = self.table[positions.long()][:, None, :]
+        return q + t, k + t
+
+
+class AttentionWithPosition(PagedAttention):
+    def tensor_specs(self):
+        return {**super().tensor_specs(), **self.position.tensor_specs()}
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig:
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    ffn: int
+    eps: float
+    max_positions: int
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d["architectures"][0], d["vocab_size"], d["hidden_size"], d["num_heads"], d["num_kv_heads"],
+                   d["head_dim"], d["ffn"], d["eps"], d["max_positions"])
+
+
+def build_toy(c: ToyConfig) -> DecoderLM:
+    def attention(i):
+        return AttentionWithPosition(f"l{i}.attn.", c.hidden_size, c.num_heads, c.num_kv_heads, c.head_dim,
+                                     LearnedAdditivePosition(f"l{i}.attn.pos", c.max_positions, c.head_dim),
+                                     qk_norm_eps=c.eps)
+
+    def block(i, mixer):
+        return PreNormBlock(RMSNorm(f"l{i}.n1", c.hidden_size, c.eps), mixer, RMSNorm(f"l{i}.n2", c.hidden_size, c.eps),
+                            GatedMLP(f"l{i}.mlp.", c.hidden_size, c.ffn))
+
+    blocks = [block(0, RunningMeanMixer("l0.mean.weight", c.hidden_size)), block(1, attention(1)), block(2, attention(2))]
+    # block 0 runs twice (its second run has state of its own); block 2 reads the keys and values of block 1
+    plan = [PlanEntry(0), PlanEntry(1), PlanEntry(0), PlanEntry(2, cache=1, writes=False)]
+    return DecoderLM(c, Embedding("emb", c.vocab_size, c.hidden_size), blocks, plan, RMSNorm("fn", c.hidden_size, c.eps),
+                     Linear(["head"], c.hidden_size, [c.vocab_size]), tied_head=False)
+
+
+def toy_plain(ids, w, c: ToyConfig):
+    T = len(ids)
+    n = lambda x, name: plain.rms_norm(x, w[name], c.eps)
+
+    def mlp(x, i):
+        return plain.gated_mlp(x, w[f"l{i}.mlp.gate_proj.weight"], w[f"l{i}.mlp.up_proj.weight"], w[f"l{i}.mlp.down_proj.weight"])
+
+    def mean_block(x):
+        xin = n(x, "l0.n1")
+        m = torch.cumsum(xin, 0) / torch.arange(1, T + 1, dtype=D)[:, None]
+        r = x + plain.linear(m, w["l0.mean.weight"])
+        return r + mlp(n(r, "l0.n2"), 0)
+
+    def qkv(x, i):
+        pos = w[f"l{i}.attn.pos"][:T][:, None, :]
+        q = plain.linear(x, w[f"l{i}.attn.q_proj.weight"]).reshape(T, c.num_heads, c.head_dim)
+        k = plain.linear(x, w[f"l{i}.attn.k_proj.weight"]).reshape(T, c.num_kv_heads, c.head_dim)
+        v = plain.linear(x, w[f"l{i}.attn.v_proj.weight"]).reshape(T, c.num_kv_heads, c.head_dim)
+        q = plain.rms_norm(q, w[f"l{i}.attn.q_norm.weight"], c.eps) + pos
+        k = plain.rms_norm(k, w[f"l{i}.attn.k_norm.weight"], c.eps) + pos
+        return q, k, v
+
+    def attn_block(x, i, kv=None):
+        q, k, v = qkv(n(x, f"l{i}.n1"), i)
+        if kv is not None:
+            k, v = kv
+        a = plain.causal_gqa_attention(q, k, v).reshape(T, -1)
+        r = x + plain.linear(a, w[f"l{i}.attn.o_proj.weight"])
+        return r + mlp(n(r, f"l{i}.n2"), i), (k, v)
+
+    h = plain.embedding(ids, w["emb"])
+    h = mean_block(h)
+    h, kv1 = attn_block(h, 1)
+    h = mean_block(h)
+    h, _ = attn_block(h, 2, kv1)
+    return plain.fast_linear(n(h, "fn"), w["head"])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_architecture_registers_builds_and_steps(dtype):
+    register_architecture("ToyForCausalLM", ToyConfig, build_toy)
+    c = ToyConfig.from_dict(dict(architectures=["ToyForCausalLM"], vocab_size=61, hidden_size=40, num_heads=4,
+                                 num_kv_heads=2, head_dim=16, ffn=56, eps=1e-5, max_positions=64))
+    model = build_toy(c)
+    ctx, w = bound(model, dtype, seed=9)
+    model.ctx = ctx
+    cache = CacheManager(model, page_size=4, num_pages=12, max_requests=3, dtype=dtype, device=ctx.device)
+    assert len(cache.groups) == 1 and cache.groups[0].cache_ids == [1]  # one cache layer, shared by two entries
+    assert sorted(cache.states) == [0, 2]  # the block that runs twice has two state rows
+    runner = ModelRunner(model, cache)
+    seqs = {"x": random_tokens(21, 61, 1), "y": random_tokens(13, 61, 2)}
+    want = {k: toy_plain(v, w, c) for k, v in seqs.items()}
+    sx, sy = runner.admit(), runner.admit()
+    got = {"x": [], "y": []}
+    # portions of x beside portions and single tokens of y
+    for (ax, bx), (ay, by) in (((0, 9), (0, 2)), ((9, 10), (2, 11)), ((10, 21), (11, 12)), ((21, 21), (12, 13))):
+        entries, names = [], []
+        if bx > ax:
+            entries.append(StepEntry(sx, seqs["x"][ax:bx], list(range(bx - ax))))
+            names.append(("x", bx - ax))
+        if by > ay:
+            entries.append(StepEntry(sy, seqs["y"][ay:by], list(range(by - ay))))
+            names.append(("y", by - ay))
+        out = runner.step(entries).cpu()
+        at = 0
+        for name, cnt in names:
+            got[name].append(out[at : at + cnt])
+            at += cnt
+    for k in seqs:
+        err = (torch.cat(got[k]).double() - want[k]).abs().max().item()
+        assert err < TOL[dtype], (k, err)
+    # a slot that is used again starts from zeroed state
+    runner.release(sx)
+    s2 = runner.admit()
+    assert s2 == sx
+    again = runner.step([StepEntry(s2, seqs["y"], list(range(13)))]).cpu()
+    assert (again.double() - want["y"]).abs().max() < TOL[dtype]
