@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Qwen3-8B layer sizes, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+
+A "step" is one decode step of the whole engine (scheduler, model step over the
+paged cache, sampling) with `batch` live requests whose context ends at
+`context` tokens.  Seeded random weights (bfloat16), uniform random token ids.
+One JSON line is printed: `value` = decoded tokens per second, `prefill` = a
+2048-token prompt in one step, `roofline` = bytes the decode step has to read
+(every weight it uses once + the cache of the live requests) / its time against
+8 TB/s, `points` = decode at batch 1 and 64.  The reference publishes nothing
+for this configuration (its only table is Qwen3-0.6B in float32 on an unnamed
+GPU, readme.md:62-66), so `vs_baseline` is null.
+"""
+import argparse
+import json
+import sys
+import time
+
+# Qwen3-8B layer sizes
+SIZES = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=36, hidden_size=4096,
+    num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
+    rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+)
+HBM_PEAK = 8.0e12  # bytes/s
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+PAGE_SIZE = 16
+PREFILL_TOKENS = 2048
+
+
+def weight_bytes_per_step(cfg, elem=2):
+    h, d = cfg.hidden_size, cfg.head_dim
+    per_layer = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d * h  # qkv
+    per_layer += h * cfg.num_attention_heads * d  # o
+    per_layer += 3 * h * cfg.intermediate_size  # gate, up, down
+    per_layer += 2 * h + 2 * d  # norms
+    return (per_layer * cfg.num_hidden_layers + h + cfg.vocab_size * h) * elem
+
+
+def kv_bytes_per_token(cfg, elem=2):
+    return 2 * cfg.num_key_value_heads * cfg.head_dim * cfg.num_hidden_layers * elem
+
+
+def prefill_flops(cfg, tokens):
+    h, d = cfg.hidden_size, cfg.head_dim
+    per_layer = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d * h + h * cfg.num_attention_heads * d
+    per_layer += 3 * h * cfg.intermediate_size
+    linear = 2.0 * tokens * per_layer * cfg.num_hidden_layers + 2.0 * cfg.vocab_size * h  # head: one row
+    attention = 4.0 * cfg.num_attention_heads * d * (tokens * (tokens + 1) / 2) * cfg.num_hidden_layers
+    return linear + attention
+
+
+def make_engine(model, batch, context, max_tokens_per_step=8192):
+    from litellmengine_amd.engine import LLMEngine
+
+    pages_each = (context + PAGE_SIZE - 1) // PAGE_SIZE + 1
+    return LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_each * batch, max_requests=batch,
+                     max_tokens_per_step=max_tokens_per_step, prefill_chunk=2048, max_pages_per_request=pages_each)
+
+
+def random_prompts(n, length, vocab, seed):
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n, length), generator=g).tolist()
+
+
+def time_decode(model, cfg, batch, context, steps, warmup):
+    """`steps` timed decode steps of `batch` requests; the last one runs at a
+    attends to `context` keys.  Returns seconds per step."""
+    import torch
+
+    engine = make_engine(model, batch, context)
+    prompt_len = context - (steps + warmup)
+    for p in random_prompts(batch, prompt_len, cfg.vocab_size, 100 + batch):
+        engine.prefill(engine.add_request(p, steps + warmup + 1))  # each prompt alone, in portions
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    lens = [r.cached_len for r in engine.scheduler.requests.values()]
+    assert all(n == context for n in lens), lens
+    return dt
+
+
+def time_prefill(model, cfg, tokens, repeats=3):
+    import torch
+
+    engine = make_engine(model, 1, tokens + 16, max_tokens_per_step=tokens)
+    best = None
+    for i in range(repeats + 1):
+        req = engine.add_request(random_prompts(1, tokens, cfg.vocab_size, 7 + i)[0], 1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()  # the whole prompt in one step, one token drawn
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert req.finished and engine.num_steps == i + 1
+        if i > 0:  # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=SIZES["num_hidden_layers"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.models import random_model
+
+    sizes = dict(SIZES, num_hidden_layers=args.layers)
+    cfg = Qwen3Config.from_dict(sizes)
+    torch.cuda.set_device(0)
+    model = random_model(cfg, seed=0, dtype=args.dtype)
+    elem = 2 if args.dtype == "bfloat16" else 4
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+
+    dt = time_decode(model, cfg, args.batch, args.context, args.steps, args.warmup)
+    value = args.batch / dt
+    avg_ctx = args.context - (args.steps - 1) / 2.0
+    step_bytes = weight_bytes_per_step(cfg, elem) + args.batch * avg_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / dt
+    line = {
+        "metric": "decode tok/s @ batch 8, Qwen3-8B sizes, context 4096 (+ prefill tok/s @ 2048, % roofline)",
+        "value": round(value, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": short,
+        "data": "synthetic: seeded random weights, uniform random token ids",
+        "config": {
+            "model": "Qwen3-8B sizes (random weights)", "layers": cfg.num_hidden_layers,
+            "layers_of_full_model": SIZES["num_hidden_layers"], "hidden": cfg.hidden_size,
+            "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": args.batch,
+            "seq_len": args.context, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS, "parallelism": "none (1 GPU)",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    if not args.no_points:
+        pt = time_prefill(model, cfg, PREFILL_TOKENS)
+        line["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                           "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MFMA_PEAK[short], 4)}
+        points = {}
+        for b in (1, 64):
+            s = max(8, args.steps // 2)
+            points[f"decode_b{b}"] = round(b / time_decode(model, cfg, b, args.context, s, 4), 2)
+        line["points"] = points
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -42,9 +42,10 @@ class LLMEngine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
-    def step(self) -> List[Request]:
-        """One scheduled step.  Returns the requests that finished in it."""
-        plan = self.scheduler.schedule()
+    def step(self, only: Optional[Sequence[int]] = None) -> List[Request]:
+        """One scheduled step (of the requests with the ids in `only`, if given).
+        Returns the requests that finished in it."""
+        plan = self.scheduler.schedule(only)
         if not plan:
             return []
         entries = [
@@ -60,6 +61,12 @@ class LLMEngine:
             parts = ", ".join(f"req {p.request.request_id}: {p.num_tokens} tok" for p in plan)
             print(f"[step {self.num_steps}] {parts}; sampled {sampled}", file=sys.stderr)
         return done
+
+    def prefill(self, request: Request) -> None:
+        """Run `request` alone until its prompt is cached and its first token drawn
+        (PagedGenerateEngine::prefill, src/engine/paged_generate_engine.cpp:99-149)."""
+        while not request.finished and (request.cached_len == 0 or request.extend_len > 1):
+            self.step(only=[request.request_id])
 
     def run_until_finished(self) -> None:
         while self.has_work():

@@ -95,9 +95,14 @@ class Scheduler:
         return bool(self.waiting or self.running)
 
     # -- one step ---------------------------------------------------------------------
-    def schedule(self) -> List[Portion]:
+    def schedule(self, only: Optional[Sequence[int]] = None) -> List[Portion]:
+        """The portions of the next step.  `only` (request ids) restricts the step to
+        those requests, the way the reference's callers prefill one request alone
+        or decode a chosen set (src/engine/paged_generate_engine.cpp:99-149, :182-341)."""
         budget = self.max_tokens_per_step
-        order = [r for r in self.running if r.extend_len == 1] + [r for r in self.running if r.extend_len > 1]
+        chosen = None if only is None else set(only)
+        mine = [r for r in self.running if chosen is None or r.request_id in chosen]
+        order = [r for r in mine if r.extend_len == 1] + [r for r in mine if r.extend_len > 1]
         plan: List[Portion] = []
         for r in order:
             if budget == 0:
@@ -116,8 +121,10 @@ class Scheduler:
             budget += sum(p.num_tokens for p in plan if p.request is victim)
             plan = [p for p in plan if p.request is not victim]
 
-        while not preempted and self.waiting and budget > 0 and self.cache.num_free_slots > 0:
-            r = self.waiting[0]
+        while not preempted and budget > 0 and self.cache.num_free_slots > 0:
+            r = next((w for w in self.waiting if chosen is None or w.request_id in chosen), None)
+            if r is None:
+                break
             n = min(r.extend_len, self.prefill_chunk, budget)
             slot = self.cache.admit()
             wants = [(p.request.slot, p.start + p.num_tokens) for p in plan] + [(slot, n)]
@@ -126,7 +133,7 @@ class Scheduler:
                 if not self.running:
                     raise OutOfPages("the first waiting request does not fit into the empty cache")
                 break
-            self.waiting.popleft()
+            self.waiting.remove(r)
             r.slot = slot
             r.status = RequestStatus.RUNNING
             r.admitted_at = self._admissions
