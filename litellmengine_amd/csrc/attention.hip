@@ -1,5 +1,5 @@
 // Paged grouped-query attention over the cache, for any mix of prompt portions
-// and single decoded tokens in one launch.
+// and single decoded tokens in one step.
 //
 // The reference has three kernels, none of which covers a prompt portion after
 // a past: flash_attention_kernel (prefill of one request over its own K/V,
@@ -12,7 +12,19 @@
 //   sees keys lo..p,  lo = max(0, p - window + 1) with a window, else 0
 //   score_j = (q . k_j) * scale;  softmax over j streamed in 32-bit (m, l, acc)
 //   kv head of q head h = h / (nq / nkv)                  (:577-668 for the maths)
-// A cache page holds [2 (K, V)][nkv][page_size][d].
+// A cache page holds K as [nkv][page_size][d], then V as [nkv][d][page_size].
+//
+// Kernels:
+//  * paged_attention_generic_kernel: any type, head size <= 256, page size,
+//    window; one workgroup per (token, q head).  The 32-bit path and odd sizes.
+//  * mfma_decode_kernel / mfma_combine_kernel: bfloat16, head size a multiple of
+//    32, page size a multiple of 16.  One workgroup per (request, kv head, key
+//    split); the q heads of the group (and up to 16 / group tokens) are the 16
+//    columns of v_mfma_f32_16x16x32_bf16 tiles, so every K/V byte is read once
+//    per group; the four wavefronts take every fourth 32-key step; partial
+//    (m, l, acc) of the splits are merged by the combine kernel.
+//  * mfma_prefill_kernel: same tile code, 32 rows (token, head) per wavefront,
+//    all keys up to each row's own position.
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -20,8 +32,6 @@ LLE_DEFINE_ERROR_STRING()
 #define ATT_WAVES 4
 #define ATT_MAX_R 4  // head_dim <= 256
 
-// One workgroup per (query token, q head); each wavefront walks every fourth
-// key, lanes split the head dimension.  Any head_dim <= 256, page size, window.
 template <typename T>
 __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
@@ -51,12 +61,13 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_k
         acc[r] = 0.f;
     }
     float m = -FLT_MAX, l = 0.f;
-    const int64_t v_off = (int64_t)nkv * page_size * d;
+    const int64_t v_base = ((int64_t)nkv + kvh) * page_size * d;
     for (int j = lo + wave; j <= pos; j += ATT_WAVES) {
         const int lp = j / page_size;
-        const int64_t page = table[lp];
-        const T* kp = kv_layer + page * page_stride + ((int64_t)kvh * page_size + (j - lp * page_size)) * d;
-        const T* vp = kp + v_off;
+        const int off = j - lp * page_size;
+        const T* page = kv_layer + (int64_t)table[lp] * page_stride;
+        const T* kp = page + ((int64_t)kvh * page_size + off) * d;
+        const T* vp = page + v_base + off;  // element e of the value row at vp[e * page_size]
         float dot = 0.f;
 #pragma unroll
         for (int r = 0; r < ATT_MAX_R; ++r) {
@@ -71,7 +82,7 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_k
 #pragma unroll
         for (int r = 0; r < ATT_MAX_R; ++r) {
             const int e = lane + LLE_WAVE * r;
-            if (e < d) acc[r] = acc[r] * alpha + beta * to_f32<T>(vp[e]);
+            if (e < d) acc[r] = acc[r] * alpha + beta * to_f32<T>(vp[(int64_t)e * page_size]);
         }
         m = new_m;
     }
@@ -114,4 +125,376 @@ extern "C" int lle_paged_attention_generic(const void* q, const void* kv_layer, 
             (const int32_t*)cu_tokens, (const int32_t*)kv_lens, (const int32_t*)token_seq, (bf16_t*)out, nq, nkv,
             d, page_size, page_stride, max_pages, window, scale);
     LLE_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------
+// matrix-core kernels (bfloat16)
+// ---------------------------------------------------------------------------------
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define NEG_BIG (-1.0e30f)
+#define KSTEP 32  // keys per step: two 16-key tiles, each inside one page
+
+// What one lane knows about the query row it serves (row = lane % 16 of a 16-row tile).
+struct RowInfo {
+    const bf16_t* q;  // start of the row's head in q, or nullptr for a row that does not exist
+    int pos;          // last key the row sees
+    int lo;           // first key the row sees
+};
+
+// One wavefront runs `RT` tiles of 16 query rows over the 32-key steps
+// step_begin, step_begin + step_stride, ... < step_end.  Products:
+//   S^T = K Q^T   (A = K tile [16 keys x 32], B = Q^T [32 x 16 rows])
+//   O^T += V^T P^T (A = V^T tile [16 d x 32 keys], B = P^T [32 keys x 16 rows])
+// With v_mfma_f32_16x16x32_bf16 a lane (c = lane / 16, r = lane % 16) holds, of a
+// result tile, column r and rows 4c..4c+3: for S^T that is query row r and keys
+// 4c..4c+3 — exactly what the B operand of the second product wants, so P never
+// leaves registers, and the softmax state of row r sits in the lanes r + 16c.
+// The k slots of the second product are (tile A keys 4c..4c+3, tile B keys 4c..4c+3).
+template <int DK, int RT>
+__device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16_t* __restrict__ kv_layer,
+                                            const int32_t* __restrict__ table, int kvh, int nkv, int P,
+                                            int64_t page_stride, int step_begin, int step_end, int step_stride,
+                                            int lo_min, int hi, float scale_log2, f32x4 (&o)[RT][2 * DK],
+                                            float (&m)[RT], float (&l)[RT]) {
+    constexpr int D = DK * 32;
+    const int lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+
+    bf16x8 qv[RT][DK];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) {
+            if (row[t].q) {
+                qv[t][ks] = *(const bf16x8*)(row[t].q + 32 * ks + 8 * c);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qv[t][ks][i] = (bf16_t)0.0f;
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < 2 * DK; ++n) o[t][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m[t] = NEG_BIG;
+        l[t] = 0.f;
+    }
+    const int64_t k_head = (int64_t)kvh * P * D;
+    const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
+
+    for (int st = step_begin; st < step_end; st += step_stride) {
+        const int j0 = st * KSTEP;
+        const bf16_t* page[2];
+        int off[2];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            const int jx = j0 + 16 * x;
+            // a tile wholly outside [lo_min, hi] may lie in a page that is not there: look up a key that is
+            const int probe = min(max(jx, lo_min), hi);
+            page[x] = kv_layer + (int64_t)table[probe / P] * page_stride;
+            off[x] = jx % P;
+        }
+        // K operands: lane (c, r16) holds key r16 of the tile, elements 32 ks + 8 c .. + 7
+        bf16x8 ka[2][DK];
+#pragma unroll
+        for (int x = 0; x < 2; ++x)
+#pragma unroll
+            for (int ks = 0; ks < DK; ++ks)
+                ka[x][ks] = *(const bf16x8*)(page[x] + k_head + (int64_t)(off[x] + r16) * D + 32 * ks + 8 * c);
+        // V^T operands: lane holds value element 16 n + r16, keys 4c..4c+3 of tile A then of tile B
+        bf16x8 va[2 * DK];
+#pragma unroll
+        for (int n = 0; n < 2 * DK; ++n) {
+            const bf16x4 a = *(const bf16x4*)(page[0] + v_head + (int64_t)(16 * n + r16) * P + off[0] + 4 * c);
+            const bf16x4 b = *(const bf16x4*)(page[1] + v_head + (int64_t)(16 * n + r16) * P + off[1] + 4 * c);
+            va[n] = bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        }
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            f32x4 s[2];
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                s[x] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < DK; ++ks)
+                    s[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[x][ks], qv[t][ks], s[x], 0, 0, 0);
+            }
+            // scores of row r16 for keys j0 + 16 x + 4 c + i
+            float sc[8];
+            bool ok[8];
+            float tile_max = NEG_BIG;
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int j = j0 + 16 * x + 4 * c + i;
+                    ok[4 * x + i] = j >= row[t].lo && j <= row[t].pos;
+                    sc[4 * x + i] = s[x][i] * scale_log2;
+                    if (ok[4 * x + i]) tile_max = fmaxf(tile_max, sc[4 * x + i]);
+                }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
+            const float new_m = fmaxf(m[t], tile_max);
+            const float alpha = exp2f(m[t] - new_m);
+            m[t] = new_m;
+            float psum = 0.f;
+            bf16x8 pb;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = ok[i] ? exp2f(sc[i] - new_m) : 0.f;
+                psum += p;
+                pb[i] = (bf16_t)p;
+            }
+            l[t] = l[t] * alpha + psum;
+#pragma unroll
+            for (int n = 0; n < 2 * DK; ++n) {
+                o[t][n] *= alpha;
+                o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[n], pb, o[t][n], 0, 0, 0);
+            }
+        }
+    }
+    // the partial sums of a row sit in the four lanes r16 + 16 c
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        l[t] += __shfl_xor(l[t], 16, LLE_WAVE);
+        l[t] += __shfl_xor(l[t], 32, LLE_WAVE);
+    }
+}
+
+// row `r` of the (token, head-in-group) rows of one request and kv head
+__device__ __forceinline__ RowInfo make_row(const bf16_t* q, int r, int nrows, int G, int q_start, int past, int nq,
+                                            int kvh, int D, int window) {
+    RowInfo info;
+    if (r < nrows) {
+        const int t = r / G, g = r - t * G;
+        info.q = q + ((int64_t)(q_start + t) * nq + kvh * G + g) * D;
+        info.pos = past + t;
+        info.lo = window > 0 ? max(0, info.pos - window + 1) : 0;
+    } else {
+        info.q = nullptr;
+        info.pos = -1;
+        info.lo = 0;
+    }
+    return info;
+}
+
+// Requests whose rows (q_len * group) fit one 16-row tile: decoded tokens and very
+// short portions.  grid = (requests, kv heads, splits).
+template <int DK>
+__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
+    float scale_log2) {
+    constexpr int D = DK * 32;
+    extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
+    float* s_o = smem;
+    float* s_m = smem + ATT_WAVES * 16 * D;
+    float* s_l = s_m + ATT_WAVES * 16;
+
+    const int s = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, nsplit = gridDim.z;
+    const int G = nq / nkv;
+    const int q_start = cu_tokens[s];
+    const int q_len = cu_tokens[s + 1] - q_start;
+    const int nrows = q_len * G;
+    if (nrows > 16) return;  // the prefill kernel's
+    const int kv_len = kv_lens[s];
+    const int past = kv_len - q_len;
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
+
+    RowInfo row[1] = {make_row(q, r16, nrows, G, q_start, past, nq, kvh, D, window)};
+    const int lo_min = window > 0 ? max(0, past - window + 1) : 0;
+    const int hi = kv_len - 1;
+    const int first = lo_min / KSTEP, last = hi / KSTEP;
+    const int per_split = (last - first + 1 + nsplit - 1) / nsplit;
+    const int sb = first + split * per_split;
+    const int se = min(last + 1, sb + per_split);
+
+    f32x4 o[1][2 * DK];
+    float m[1], l[1];
+    attend_rows<DK, 1>(row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, ATT_WAVES, lo_min, hi,
+                       scale_log2, o, m, l);
+
+    // merge the four wavefronts
+#pragma unroll
+    for (int n = 0; n < 2 * DK; ++n)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_o[(wave * 16 + r16) * D + 16 * n + 4 * c + i] = o[0][n][i];
+    if (c == 0) {
+        s_m[wave * 16 + r16] = m[0];
+        s_l[wave * 16 + r16] = l[0];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
+        const int r = idx / D, e = idx - r * D;
+        float big = s_m[r];
+#pragma unroll
+        for (int w = 1; w < ATT_WAVES; ++w) big = fmaxf(big, s_m[w * 16 + r]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < ATT_WAVES; ++w) {
+            const float f = exp2f(s_m[w * 16 + r] - big);
+            num += s_o[(w * 16 + r) * D + e] * f;
+            den += s_l[w * 16 + r] * f;
+        }
+        const int t = r / G, g = r - t * G;
+        const int64_t head_row = (int64_t)(q_start + t) * nq + kvh * G + g;
+        if (nsplit == 1) {
+            out[head_row * D + e] = (bf16_t)(num / den);
+        } else {
+            ws_o[(head_row * nsplit + split) * D + e] = num;
+            if (e == 0) {
+                ws_ml[(head_row * nsplit + split) * 2] = big;
+                ws_ml[(head_row * nsplit + split) * 2 + 1] = den;
+            }
+        }
+    }
+}
+
+// merges the splits of mfma_decode_kernel.  grid = (tokens, q heads), 64 threads.
+__global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __restrict__ ws_o,
+                                                                const float* __restrict__ ws_ml,
+                                                                const int32_t* __restrict__ cu_tokens,
+                                                                const int32_t* __restrict__ token_seq,
+                                                                bf16_t* __restrict__ out, int nq, int nkv, int D,
+                                                                int nsplit) {
+    const int64_t tok = blockIdx.x;
+    const int h = blockIdx.y;
+    const int s = token_seq[tok];
+    if ((cu_tokens[s + 1] - cu_tokens[s]) * (nq / nkv) > 16) return;
+    const int64_t head_row = tok * nq + h;
+    const float* ml = ws_ml + head_row * nsplit * 2;
+    float big = NEG_BIG;
+    for (int k = 0; k < nsplit; ++k) big = fmaxf(big, ml[2 * k]);
+    float den = 0.f;
+    for (int k = 0; k < nsplit; ++k) den += ml[2 * k + 1] * exp2f(ml[2 * k] - big);
+    for (int e = threadIdx.x; e < D; e += blockDim.x) {
+        float num = 0.f;
+        for (int k = 0; k < nsplit; ++k) num += ws_o[(head_row * nsplit + k) * D + e] * exp2f(ml[2 * k] - big);
+        out[head_row * D + e] = (bf16_t)(num / den);
+    }
+}
+
+// Requests with more than 16 rows.  grid = (row blocks of 128, kv heads, requests);
+// each wavefront owns 32 rows and walks all keys up to its last row's position.
+#define PRE_RT 2
+template <int DK>
+__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_prefill_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, int nq, int nkv, int P, int64_t page_stride,
+    int max_pages, int window, float scale_log2) {
+    constexpr int D = DK * 32;
+    const int s = blockIdx.z, kvh = blockIdx.y;
+    const int G = nq / nkv;
+    const int q_start = cu_tokens[s];
+    const int q_len = cu_tokens[s + 1] - q_start;
+    const int nrows = q_len * G;
+    if (nrows <= 16) return;  // the decode kernel's
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    const int row0 = (blockIdx.x * ATT_WAVES + wave) * (16 * PRE_RT);
+    if (row0 >= nrows) return;
+    const int kv_len = kv_lens[s];
+    const int past = kv_len - q_len;
+    const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
+
+    RowInfo row[PRE_RT];
+#pragma unroll
+    for (int t = 0; t < PRE_RT; ++t) row[t] = make_row(q, row0 + 16 * t + r16, nrows, G, q_start, past, nq, kvh, D, window);
+    const int first_pos = past + row0 / G;
+    const int last_row = min(nrows, row0 + 16 * PRE_RT) - 1;
+    const int hi = past + last_row / G;
+    const int lo_min = window > 0 ? max(0, first_pos - window + 1) : 0;
+
+    f32x4 o[PRE_RT][2 * DK];
+    float m[PRE_RT], l[PRE_RT];
+    attend_rows<DK, PRE_RT>(row, kv_layer, table, kvh, nkv, P, page_stride, lo_min / KSTEP, hi / KSTEP + 1, 1,
+                            lo_min, hi, scale_log2, o, m, l);
+#pragma unroll
+    for (int t = 0; t < PRE_RT; ++t) {
+        const int r = row0 + 16 * t + r16;
+        if (r >= nrows) continue;
+        const int tk = r / G, g = r - tk * G;
+        bf16_t* dst = out + ((int64_t)(q_start + tk) * nq + kvh * G + g) * D;
+        const float inv = 1.0f / l[t];
+#pragma unroll
+        for (int n = 0; n < 2 * DK; ++n) {
+            bf16x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[t][n][i] * inv);
+            *(bf16x4*)(dst + 16 * n + 4 * c) = v;
+        }
+    }
+}
+
+template <int DK>
+static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* block_tables,
+                       const int32_t* seq_slots, const int32_t* cu_tokens, const int32_t* kv_lens,
+                       const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
+                       int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
+                       int run_decode, int nsplit, int run_prefill, int max_q_len, hipStream_t stream) {
+    constexpr int D = DK * 32;
+    const int G = nq / nkv;
+    if (run_decode) {
+        const size_t smem = (size_t)(ATT_WAVES * 16 * D + 2 * ATT_WAVES * 16) * sizeof(float);
+        if (smem > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void*)mfma_decode_kernel<DK>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return (int)e;
+        }
+        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit), ATT_WAVES * LLE_WAVE, smem, stream>>>(
+            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, nq, nkv, P, page_stride,
+            max_pages, window, scale_log2);
+        if (nsplit > 1)
+            mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(ws_o, ws_ml, cu_tokens, token_seq, out, nq, nkv,
+                                                                      D, nsplit);
+    }
+    if (run_prefill) {
+        const int rows = max_q_len * G;
+        const int blocks = (rows + ATT_WAVES * 16 * PRE_RT - 1) / (ATT_WAVES * 16 * PRE_RT);
+        mfma_prefill_kernel<DK><<<dim3(blocks, nkv, S), ATT_WAVES * LLE_WAVE, 0, stream>>>(
+            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, nq, nkv, P, page_stride, max_pages, window,
+            scale_log2);
+    }
+    return (int)hipGetLastError();
+}
+
+// bfloat16, head_dim a multiple of 32 (<= 256), page size a multiple of 16.
+// run_decode / run_prefill say which kinds of request the batch holds (requests
+// with q_len * group <= 16 rows are the decode kernel's); nsplit > 1 needs the
+// workspaces ws_o [N * nq * nsplit * d] and ws_ml [N * nq * nsplit * 2] floats.
+extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, const void* block_tables,
+                                        const void* seq_slots, const void* cu_tokens, const void* kv_lens,
+                                        const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
+                                        int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
+                                        int window, float scale, int run_decode, int nsplit, int run_prefill,
+                                        int max_q_len, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
+    if (S > 65535 || nkv > 65535) return (int)hipErrorInvalidValue;
+    const float scale_log2 = scale * 1.44269504088896340736f;
+#define LLE_ATT_CASE(DKV)                                                                                          \
+    case DKV:                                                                                                      \
+        return launch_mfma<DKV>((const bf16_t*)q, (const bf16_t*)kv_layer, (const int32_t*)block_tables,            \
+                                (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
+                                (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
+                                page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit,          \
+                                run_prefill, max_q_len, stream);
+    switch (d / 32) {
+        LLE_ATT_CASE(1)
+        LLE_ATT_CASE(2)
+        LLE_ATT_CASE(3)
+        LLE_ATT_CASE(4)
+        LLE_ATT_CASE(5)
+        LLE_ATT_CASE(6)
+        LLE_ATT_CASE(7)
+        LLE_ATT_CASE(8)
+    }
+#undef LLE_ATT_CASE
+    return (int)hipErrorInvalidValue;
 }

@@ -177,9 +177,13 @@ class HipOps:
         return q_out
 
     def paged_attention(self, q, kv_layer, block_table, seq_slots, cu_tokens, kv_lens, token_seq,
-                        window: Optional[int], scale: float, max_q_len: int = 0, max_kv_len: int = 0) -> torch.Tensor:
-        """q [N, nq, d] against the pages -> [N, nq * d].  `max_q_len`/`max_kv_len`
-        are host-side bounds of this batch (hints for choosing a kernel)."""
+                        window: Optional[int], scale: float, min_q_len: int = 0, max_q_len: int = 0,
+                        max_kv_len: int = 0) -> torch.Tensor:
+        """q [N, nq, d] against the pages -> [N, nq * d].  `min_q_len`, `max_q_len`
+        and `max_kv_len` are host-side bounds of this batch; they choose the kernels
+        and the number of key splits, never the result.  bfloat16 with head_dim a
+        multiple of 32 and a page size a multiple of 16 runs on the matrix cores;
+        everything else takes the generic kernel."""
         _dev(q, "q")
         _dev(kv_layer, "kv_layer", q.dtype)
         for t, name in ((block_table, "block_table"), (seq_slots, "seq_slots"), (cu_tokens, "cu_tokens"),
@@ -195,12 +199,46 @@ class HipOps:
         _need(cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "cu_tokens [S + 1], kv_lens [S]")
         _need(block_table.dim() == 2, "block_table must be [slots, pages]")
         out = torch.empty((N, nq * d), dtype=q.dtype, device=q.device)
-        self._run("attention", "lle_paged_attention_generic",
-                  [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P],
+        win = int(window) if window else 0
+        mfma = (q.dtype == torch.bfloat16 and d % 32 == 0 and page_size % 16 == 0 and max_q_len > 0
+                and max_kv_len > 0 and S <= 65535 and not self.force_generic_attention)
+        if not mfma:
+            self._run("attention", "lle_paged_attention_generic",
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P],
+                      _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
+                      _ptr(token_seq), _ptr(out), N, nq, nkv, d, page_size, kv_layer.stride(0), block_table.shape[1],
+                      win, float(scale), dtype_code(q.dtype))
+            return out
+        group = nq // nkv
+        min_q_len = min_q_len or 1
+        run_decode = min_q_len * group <= 16
+        run_prefill = max_q_len * group > 16
+        nsplit, ws_o, ws_ml = 1, None, None
+        if run_decode:
+            nsplit = self.decode_splits(S, nkv, max_kv_len, win)
+            if nsplit > 1:
+                ws_o = torch.empty((N * nq * nsplit * d,), dtype=torch.float32, device=q.device)
+                ws_ml = torch.empty((N * nq * nsplit * 2,), dtype=torch.float32, device=q.device)
+        self._run("attention", "lle_paged_attention_mfma",
+                  [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _I, _I, _P],
                   _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
-                  _ptr(token_seq), _ptr(out), N, nq, nkv, d, page_size, kv_layer.stride(0), block_table.shape[1],
-                  int(window) if window else 0, float(scale), dtype_code(q.dtype))
+                  _ptr(token_seq), _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size,
+                  kv_layer.stride(0), block_table.shape[1], win, float(scale), int(run_decode), nsplit,
+                  int(run_prefill), max_q_len)
         return out
+
+    force_generic_attention = False  # tests flip this to compare the two families of kernels
+    DECODE_TARGET_BLOCKS = 1024
+    DECODE_MIN_STEPS_PER_SPLIT = 4  # one 32-key step per wavefront
+
+    def decode_splits(self, num_seqs: int, num_kv_heads: int, max_kv_len: int, window: int) -> int:
+        """Key splits of the decode kernel: enough workgroups to fill the chip, but
+        at least DECODE_MIN_STEPS_PER_SPLIT 32-key steps each."""
+        span = min(max_kv_len, window + 32) if window else max_kv_len
+        steps = (span + 31) // 32 + (1 if window else 0)
+        by_work = max(1, steps // self.DECODE_MIN_STEPS_PER_SPLIT)
+        by_fill = max(1, self.DECODE_TARGET_BLOCKS // max(1, num_seqs * num_kv_heads))
+        return int(min(by_work, by_fill, 64))
 
     # -- feed-forward --------------------------------------------------------------
     def silu_mul(self, gate_up) -> torch.Tensor:

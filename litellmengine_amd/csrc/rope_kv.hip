@@ -10,7 +10,9 @@
 //   v head:  copy                               -> V page of the token's slot
 // Rotation pairs element i with i + rot/2 (half split) for i < rot/2; elements
 // >= rot pass through.  angle = float(pos) * inv_freq[i], all in 32-bit.
-// A cache page holds [2 (K, V)][nkv][page_size][d]; slot = page * page_size + offset;
+// A cache page holds K as [nkv][page_size][d] and then V as [nkv][d][page_size]
+// (V is kept transposed so that the matrix-core attention kernels find the keys
+// of one value column next to each other); slot = page * page_size + offset;
 // slot < 0 skips the write.
 #include "common.h"
 
@@ -40,13 +42,13 @@ __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
         const int kvh = is_k ? head - nq : head - nq - nkv;
         const int64_t page = slot / page_size;
         const int off = slot - (int)page * page_size;
-        dst = kv_layer + page * page_stride + (int64_t)(is_k ? 0 : nkv) * page_size * d +
-              ((int64_t)kvh * page_size + off) * d;
-    }
-
-    if (!is_q && !is_k) {  // v: plain copy
-        for (int i = lane; i < d; i += LLE_WAVE) dst[i] = src[i];
-        return;
+        T* page_base = kv_layer + page * page_stride;
+        if (!is_k) {  // v: copy into the transposed page, element i of the head at [i][off]
+            T* v = page_base + ((int64_t)nkv + kvh) * page_size * d + off;
+            for (int i = lane; i < d; i += LLE_WAVE) v[(int64_t)i * page_size] = src[i];
+            return;
+        }
+        dst = page_base + ((int64_t)kvh * page_size + off) * d;
     }
 
     const void* w = is_q ? q_weight : k_weight;

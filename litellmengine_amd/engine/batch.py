@@ -44,6 +44,7 @@ class StepState:
     cu_tokens: torch.Tensor  # int32 [S + 1] first row of each request, then N
     kv_lens: torch.Tensor  # int32 [S] cached length of each request after this step
     logit_rows: torch.Tensor  # int32 [R] rows whose logits are wanted
+    min_q_len: int
     max_q_len: int
     max_kv_len: int
     seqs: List[SeqInfo]  # the same on the host
@@ -112,6 +113,7 @@ def build_step(entries: Sequence[StepEntry], cache, vocab_size: int, device) -> 
         cu_tokens=take(S + 1),
         kv_lens=take(S),
         logit_rows=take(R),
+        min_q_len=min(q.q_len for q in seqs),
         max_q_len=max(q.q_len for q in seqs),
         max_kv_len=max(kv_lens),
         seqs=seqs,

@@ -104,6 +104,6 @@ class PagedAttention(Mixer):
             )
         a = ops.paged_attention(
             q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens, step.token_seq,
-            self.window, self.scale, step.max_q_len, step.max_kv_len,
+            self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
         )
         return self.o.forward(a)

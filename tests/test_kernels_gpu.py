@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from tests.torch_ops import TorchOps
+from tests.torch_ops import TorchOps, v_pages
 
 pytestmark = pytest.mark.gpu
 
@@ -189,7 +189,7 @@ def attention_case(dtype, nq, nkv, d, P, window, lens, seed=12, pages=40, max_pa
     q = rnd((N, nq, d), dtype, seed + 2)
     i32 = lambda v: torch.tensor(v, dtype=torch.int32).cuda()
     args = (q, kv, table.cuda(), i32(slots), i32(cu), i32(kv_lens), i32(token_seq), window, 1.0 / math.sqrt(d))
-    return args, max(l for _, l in lens), max(kv_lens)
+    return args, (min(l for _, l in lens), max(l for _, l in lens)), max(kv_lens)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -198,18 +198,60 @@ def attention_case(dtype, nq, nkv, d, P, window, lens, seed=12, pages=40, max_pa
 def test_paged_attention(dtype, nq, nkv, d, P, window):
     lens = [(0, 9), (17, 1), (30, 2), (5, 11)]
     args, mq, mk = attention_case(dtype, nq, nkv, d, P, window, lens)
-    got = ops().paged_attention(*args, mq, mk)
+    got = ops().paged_attention(*args, *mq, mk)
     want = REF.paged_attention(*args)
     assert (got.double() - want.double()).abs().max() < tol(dtype, 2)
+
+
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 32, 16, None), (16, 2, 64, 32, None),
+                                               (6, 1, 96, 16, 40), (8, 2, 256, 16, None), (32, 8, 128, 16, 700),
+                                               (3, 1, 160, 48, None)])
+@pytest.mark.parametrize("lens", [
+    [(0, 9), (17, 1), (30, 2), (5, 11)],          # portions beside decoded tokens
+    [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
+    [(0, 150), (100, 70)],                        # prompt portions only, one after a past
+    [(1200, 3), (64, 64), (15, 1)],
+])
+def test_matrix_core_attention(nq, nkv, d, P, window, lens):
+    """The bfloat16 matrix-core kernels against the plain form and the generic kernel."""
+    need = max((p + l + P - 1) // P for p, l in lens)
+    args, mq, mk = attention_case(torch.bfloat16, nq, nkv, d, P, window, lens, pages=sum((p + l + P - 1) // P for p, l in lens) + 3,
+                                  max_pages=need + 1)
+    o = ops()
+    got = o.paged_attention(*args, *mq, mk)
+    want = REF.paged_attention(*args)
+    err = (got.double() - want.double()).abs().max().item()
+    assert err < 2e-2, err
+    o.force_generic_attention = True
+    try:
+        generic = o.paged_attention(*args, *mq, mk)
+    finally:
+        o.force_generic_attention = False
+    assert (got.double() - generic.double()).abs().max() < 2e-2
+
+
+def test_matrix_core_attention_far_key_and_window_edge():
+    """A key hundreds of positions back is made to dominate, with the window
+    ending exactly on it (seen) or one short of it (not seen)."""
+    nq, nkv, d, P = 8, 2, 128, 16
+    for window, seen in ((None, True), (1000 - 37, True), (1000 - 38, False)):
+        args, mq, mk = attention_case(torch.bfloat16, nq, nkv, d, P, window, [(999, 1)], pages=70, max_pages=64)
+        q, kv, table, slots = args[0], args[1], args[2], args[3]
+        far = 37
+        page, off = int(table[int(slots[0]), far // P]), far % P
+        kv[page, 0, 0, off, :] = q[0, 2] * 4.0  # q head 2 belongs to kv head 0
+        got = ops().paged_attention(*args, *mq, mk).reshape(1, nq, d)
+        hit = torch.allclose(got[0, 2].float(), v_pages(kv)[page, 0, :, off].float(), atol=2e-2)
+        assert hit == seen, (window, hit)
 
 
 def test_attention_single_token_returns_value():
     # tests/test_attention.cpp:220-281: one token sees only itself, out == V
     args, mq, mk = attention_case(torch.float32, 4, 2, 16, 4, None, [(0, 1)])
-    got = ops().paged_attention(*args, mq, mk).reshape(1, 4, 16)
+    got = ops().paged_attention(*args, *mq, mk).reshape(1, 4, 16)
     q, kv, table, slots = args[0], args[1], args[2], args[3]
     page = int(table[int(slots[0]), 0])
-    v = kv[page, 1, :, 0, :]  # [nkv, d]
+    v = v_pages(kv)[page, :, :, 0]  # [nkv, d]
     assert torch.allclose(got[0], v.repeat_interleave(2, dim=0), atol=1e-6)
 
 
@@ -221,8 +263,8 @@ def test_attention_far_key_stands_out():
     far = 37
     page, off = int(table[int(slots[0]), far // P]), far % P
     kv[page, 0, 0, off, :] = q[0, 0] * 50.0
-    got = ops().paged_attention(*args, mq, mk).reshape(1, nq, d)
-    assert torch.allclose(got[0, 0], kv[page, 1, 0, off, :], atol=1e-4)
+    got = ops().paged_attention(*args, *mq, mk).reshape(1, nq, d)
+    assert torch.allclose(got[0, 0], v_pages(kv)[page, 0, :, off], atol=1e-4)
 
 
 @pytest.mark.parametrize("V", [7, 503, 151936])

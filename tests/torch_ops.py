@@ -13,6 +13,12 @@ from typing import Optional
 import torch
 
 
+def v_pages(kv_layer):
+    """The value half of the pages [pages, 2, nkv, P, d]: stored transposed, [pages, nkv, d, P]."""
+    pages, _, nkv, P, d = kv_layer.shape
+    return kv_layer[:, 1].reshape(pages, nkv, d, P)
+
+
 class TorchOps:
     def __init__(self, compute_dtype=torch.float64):
         self.cd = compute_dtype
@@ -74,11 +80,11 @@ class TorchOps:
                     continue
                 page, off = slot // P, slot % P
                 kv_layer[page, 0, :, off, :] = k[n].to(kv_layer.dtype)
-                kv_layer[page, 1, :, off, :] = v[n].to(kv_layer.dtype)
+                v_pages(kv_layer)[page, :, :, off] = v[n].to(kv_layer.dtype)
         return q.to(qkv.dtype).contiguous()
 
     def paged_attention(self, q, kv_layer, block_table, seq_slots, cu_tokens, kv_lens, token_seq, window, scale,
-                        max_q_len=0, max_kv_len=0):
+                        min_q_len=0, max_q_len=0, max_kv_len=0):
         N, nq, d = q.shape
         nkv, P = kv_layer.shape[2], kv_layer.shape[3]
         group = nq // nkv
@@ -95,7 +101,7 @@ class TorchOps:
                 assert int(pages.min()) >= 0, "attention reads a page that was given back"
                 offs = (idx % P).long()
                 keys = kv_layer[pages, 0, :, offs, :].to(self.cd)  # [n, nkv, d]
-                vals = kv_layer[pages, 1, :, offs, :].to(self.cd)
+                vals = v_pages(kv_layer)[pages, :, :, offs].to(self.cd)  # [n, nkv, d]
                 keys = keys.repeat_interleave(group, dim=1)
                 vals = vals.repeat_interleave(group, dim=1)
                 sc = torch.einsum("hd,nhd->hn", q[t].to(self.cd), keys) * scale
