@@ -124,20 +124,29 @@ class HipOps:
     # -- matrix products -------------------------------------------------------
     def linear(self, x, weight, out_dtype=None) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
-        kernel (a true 32-bit product); bfloat16 operands with a bfloat16 result go
-        to the library product, with a float32 result to the 32-bit-accumulate kernel."""
+        kernel (a true 32-bit product).  bfloat16 operands: up to SKINNY_MAX_ROWS rows
+        the weight-streaming matrix-core kernel (either result type); more rows go to
+        the library product (bfloat16 result) or the 32-bit-accumulate kernel."""
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape
         N = weight.shape[0]
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
         out_dtype = out_dtype or x.dtype
+        if x.dtype == torch.bfloat16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0 and not self.force_library_gemm:
+            out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
+                      _ptr(x), _ptr(weight), _ptr(out), M, N, K, dtype_code(out_dtype))
+            return out
         if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
             return torch.mm(x, weight.t())
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
+
+    SKINNY_MAX_ROWS = 16  # up to here the weight-streaming kernel; above, the library product
+    force_library_gemm = False
 
     # -- attention ---------------------------------------------------------------
     def qk_norm_rope_write(self, qkv, positions, slots, q_weight, k_weight, inv_freq, rotary_dim: int,

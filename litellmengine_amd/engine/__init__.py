@@ -1,4 +1,4 @@
-from .batch import SeqInfo, StepEntry, StepState, build_step
+from .batch import SeqInfo, StepEntry, StepLayout, StepState, build_step, layout_step
 from .llm_engine import LLMEngine
 from .request import Request, RequestStatus
 from .runner import ModelRunner

@@ -53,7 +53,7 @@ class LLMEngine:
                       [p.num_tokens - 1] if p.samples else [])
             for p in plan
         ]
-        logits = self.runner.step(entries)
+        logits = self.runner.step(entries, borrow=True)
         sampled = self.sampler.pick(logits, [p.request for p in plan if p.samples])
         done = self.scheduler.update(plan, sampled)
         self.num_steps += 1

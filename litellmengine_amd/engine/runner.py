@@ -8,24 +8,46 @@ from the cache that earlier steps left, and returns float32 logits at the
 wanted places only.  Order inside a step as in the reference: the step's K/V
 are written to their pages first, then every token attends through the block
 table (src/model/qwen3.cpp:464-481 before :498-557).
+
+Steps that hold single tokens only (decoding) are launch-bound, so they are
+captured once per (batch size, context bucket) into a HIP graph and replayed:
+the step's integer arrays are copied into the graph's fixed buffer, the block
+tables are updated outside the graph, and the same kernels run.  Models whose
+mixers need the host-side view of the batch are stepped without graphs.
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from ..cache import CacheManager
-from .batch import StepEntry, StepState, build_step
+from .batch import StepEntry, StepLayout, StepState, apply_table_updates, build_step, layout_step, state_on
+
+
+class _DecodeGraph:
+    def __init__(self, graph, buf, logits):
+        self.graph = graph
+        self.buf = buf
+        self.logits = logits
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager):
+    MAX_GRAPH_BATCH = 256
+    MIN_CONTEXT_BUCKET = 256
+
+    def __init__(self, model, cache: CacheManager, use_graphs: Optional[bool] = None):
         self.model = model
         self.cache = cache
         self.device = cache.device
         self.vocab_size = model.vocab_size
         self.last_step: Optional[StepState] = None
+        graph_safe = all(getattr(b.mixer, "graph_safe", False) for b in model.blocks)
+        if use_graphs is None:
+            use_graphs = self.device.type == "cuda"
+        self.use_graphs = bool(use_graphs) and graph_safe and self.device.type == "cuda"
+        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._graph_pool = None
 
     # requests ------------------------------------------------------------------
     def admit(self) -> int:
@@ -54,17 +76,64 @@ class ModelRunner:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"wanted place {w} outside the entry's {len(e.tokens)} tokens")
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], borrow: bool = False) -> torch.Tensor:
         """Run the entries as one batch.  Returns float32 logits [wanted, vocab] in
         the order of the entries and of their `want`.  Raises cache.OutOfPages,
-        with nothing changed, when the pages for this step are not there."""
+        with nothing changed, when the pages for this step are not there.  With
+        `borrow` the result may alias memory that the next step overwrites."""
         self.check(entries)
         cache = self.cache
         wants = [(e.slot, cache.length(e.slot) + len(e.tokens)) for e in entries]
         cache.extend_many(wants)
-        state = build_step(entries, cache, self.vocab_size, self.device)
-        self.last_step = state
-        logits = self.model.forward(state, cache)
+        if self.use_graphs and len(entries) <= self.MAX_GRAPH_BATCH and all(len(e.tokens) == 1 for e in entries):
+            logits = self._graph_step(entries, borrow)
+        else:
+            state = build_step(entries, cache, self.device)
+            self.last_step = state
+            logits = self.model.forward(state, cache)
         for slot, new_len in wants:
             cache.commit(slot, new_len)
         return logits
+
+    # decoding through a captured graph ---------------------------------------------------
+    def _graph_step(self, entries: Sequence[StepEntry], borrow: bool) -> torch.Tensor:
+        cache = self.cache
+        layout = layout_step(entries, cache, all_rows=True)
+        apply_table_updates(cache, self.device)
+        bucket = self.MIN_CONTEXT_BUCKET
+        while bucket < layout.max_kv_len:
+            bucket *= 2
+        host = torch.tensor(layout.flat, dtype=torch.int32)
+        key = (layout.num_seqs, bucket)
+        g = self._graphs.get(key)
+        if g is None:
+            g = self._capture(layout, host, bucket)
+            self._graphs[key] = g
+        else:
+            g.buf.copy_(host)
+        # the slot mappings of the groups must point into this graph's buffer while it runs
+        g.graph.replay()
+        logits = g.logits
+        rows = [i for i, e in enumerate(entries) if len(e.want) > 0]
+        if len(rows) != len(entries):
+            return logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows else logits[:0].clone()
+        return logits if borrow else logits.clone()
+
+    def _capture(self, layout: StepLayout, host: torch.Tensor, bucket: int) -> _DecodeGraph:
+        buf = host.to(self.device)
+        state = state_on(buf, layout, self.cache, max_kv_len=bucket, with_seqs=False)
+        # run the step for real first (twice: library workspaces and lazy kernel set-up happen here);
+        # a decode step is idempotent: it writes the same K/V and yields the same logits
+        side = torch.cuda.Stream(device=self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                self.model.forward(state, self.cache)
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, pool=self._graph_pool):
+            logits = self.model.forward(state, self.cache)
+        if self._graph_pool is None:
+            self._graph_pool = graph.pool()
+        return _DecodeGraph(graph, buf, logits)

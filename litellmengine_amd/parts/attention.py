@@ -24,6 +24,8 @@ from .linear import Linear
 
 
 class PagedAttention(Mixer):
+    graph_safe = True
+
     def __init__(
         self,
         prefix: str,

@@ -86,6 +86,11 @@ class Mixer(Part):
     of the plan entry being run (pages of its group, the state rows, and whether
     this entry writes)."""
 
+    # True if forward() uses only device arrays of the step (no host-side view of
+    # the batch, no sizes that depend on the step's values): decode steps of such
+    # mixers may be captured into a graph and replayed.
+    graph_safe = False
+
     def cache_spec(self) -> Optional[KVCacheSpec]:
         return None
 

@@ -45,3 +45,41 @@ def test_cuts_match_plain(tmp_path, which, dtype):
         err = (got.double() - want).abs().max().item()
         assert err < TOL[dtype], (cuts, err)
     assert all(g.pool.num_held == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(tmp_path, dtype):
+    """Decode steps through a captured graph, replayed many times with eager work
+    (prompt portions of other requests, table updates) between the replays, against
+    the same steps run without graphs."""
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    seqs = [random_tokens(n, cfg["vocab_size"], 50 + i) for i, n in enumerate((61, 50, 80))]
+    outs = {}
+    for use_graphs in (True, False):
+        model = load_model(d, dtype)
+        cache = CacheManager(model, page_size=16, num_pages=40, max_requests=4, dtype=model.ctx.dtype,
+                             device=model.ctx.device)
+        runner = ModelRunner(model, cache, use_graphs=use_graphs)
+        assert runner.use_graphs == use_graphs
+        slots = [runner.admit() for _ in seqs]
+        got = []
+        runner.step([StepEntry(slots[0], seqs[0][:20]), StepEntry(slots[1], seqs[1][:9])])
+        at = [20, 9, 0]
+        for it in range(31):
+            entries = [StepEntry(slots[i], [seqs[i][at[i]]], [0]) for i in (0, 1)]
+            got.append(runner.step(entries).cpu())  # a decode step of two requests
+            at[0] += 1
+            at[1] += 1
+            if it % 3 == 0 and at[2] < 70:  # eager work between the replays
+                runner.step([StepEntry(slots[2], seqs[2][at[2] : at[2] + 7])])
+                at[2] += 7
+            if it == 20:  # three decoding rows: another graph
+                got.append(runner.step([StepEntry(slots[i], [seqs[i][at[i]]], [0]) for i in (0, 1, 2)]).cpu())
+                at = [a + 1 for a in at]
+        if use_graphs:
+            assert len(runner._graphs) >= 2
+        outs[use_graphs] = torch.cat(got)
+    assert (outs[True] - outs[False]).abs().max() < TOL[dtype] / 4
+    want = plain.model_logits_fast(seqs[0], w, cfg)
+    assert (outs[True][0].double() - want[20]).abs().max() < TOL[dtype]
