@@ -164,6 +164,7 @@ __device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16
     const int c = lane / 16, r16 = lane % 16;
 
     bf16x8 qv[RT][DK];
+    int open_lo[RT], open_hi[RT];  // steps with open_lo <= j0 and j0 + 31 <= open_hi need no mask
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
 #pragma unroll
@@ -179,6 +180,14 @@ __device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16
         for (int n = 0; n < 2 * DK; ++n) o[t][n] = f32x4{0.f, 0.f, 0.f, 0.f};
         m[t] = NEG_BIG;
         l[t] = 0.f;
+        int lo_max = row[t].q ? row[t].lo : 0, pos_min = row[t].q ? row[t].pos : 0x7fffffff;
+#pragma unroll
+        for (int off = 1; off < LLE_WAVE; off <<= 1) {
+            lo_max = max(lo_max, __shfl_xor(lo_max, off, LLE_WAVE));
+            pos_min = min(pos_min, __shfl_xor(pos_min, off, LLE_WAVE));
+        }
+        open_lo[t] = lo_max;
+        open_hi[t] = pos_min == 0x7fffffff ? -1 : pos_min;
     }
     const int64_t k_head = (int64_t)kvh * P * D;
     const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
@@ -203,13 +212,12 @@ __device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16
             for (int ks = 0; ks < DK; ++ks)
                 ka[x][ks] = *(const bf16x8*)(page[x] + k_head + (int64_t)(off[x] + r16) * D + 32 * ks + 8 * c);
         // V^T operands: lane holds value element 16 n + r16, keys 4c..4c+3 of tile A then of tile B
-        bf16x8 va[2 * DK];
+        bf16x4 va[2 * DK][2];
 #pragma unroll
-        for (int n = 0; n < 2 * DK; ++n) {
-            const bf16x4 a = *(const bf16x4*)(page[0] + v_head + (int64_t)(16 * n + r16) * P + off[0] + 4 * c);
-            const bf16x4 b = *(const bf16x4*)(page[1] + v_head + (int64_t)(16 * n + r16) * P + off[1] + 4 * c);
-            va[n] = bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-        }
+        for (int n = 0; n < 2 * DK; ++n)
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+                va[n][x] = *(const bf16x4*)(page[x] + v_head + (int64_t)(16 * n + r16) * P + off[x] + 4 * c);
 #pragma unroll
         for (int t = 0; t < RT; ++t) {
             f32x4 s[2];
@@ -220,37 +228,44 @@ __device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16
                 for (int ks = 0; ks < DK; ++ks)
                     s[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[x][ks], qv[t][ks], s[x], 0, 0, 0);
             }
-            // scores of row r16 for keys j0 + 16 x + 4 c + i
+            // scores of row r16 for keys j0 + 16 x + 4 c + i, in the base-2 domain
             float sc[8];
-            bool ok[8];
-            float tile_max = NEG_BIG;
 #pragma unroll
-            for (int x = 0; x < 2; ++x)
+            for (int i = 0; i < 8; ++i) sc[i] = s[i / 4][i % 4] * scale_log2;
+            if (!(j0 >= open_lo[t] && j0 + KSTEP - 1 <= open_hi[t])) {  // same for the whole wavefront
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int j = j0 + 16 * x + 4 * c + i;
-                    ok[4 * x + i] = j >= row[t].lo && j <= row[t].pos;
-                    sc[4 * x + i] = s[x][i] * scale_log2;
-                    if (ok[4 * x + i]) tile_max = fmaxf(tile_max, sc[4 * x + i]);
+                for (int i = 0; i < 8; ++i) {
+                    const int j = j0 + 16 * (i / 4) + 4 * c + (i % 4);
+                    if (j < row[t].lo || j > row[t].pos) sc[i] = NEG_BIG;
                 }
+            }
+            float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                   fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
             const float new_m = fmaxf(m[t], tile_max);
-            const float alpha = exp2f(m[t] - new_m);
+            // a masked score is NEG_BIG; while the row has seen no key yet new_m is NEG_BIG too,
+            // and exp2(0) = 1 would count the masked key: shift such rows so that they give 0
+            const float base = new_m <= NEG_BIG ? 0.f : new_m;
+            const float alpha = __builtin_amdgcn_exp2f(m[t] - base);
             m[t] = new_m;
             float psum = 0.f;
             bf16x8 pb;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float p = ok[i] ? exp2f(sc[i] - new_m) : 0.f;
+                const float p = __builtin_amdgcn_exp2f(sc[i] - base);
                 psum += p;
                 pb[i] = (bf16_t)p;
             }
             l[t] = l[t] * alpha + psum;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum moved somewhere
+#pragma unroll
+                for (int n = 0; n < 2 * DK; ++n) o[t][n] *= alpha;
+            }
 #pragma unroll
             for (int n = 0; n < 2 * DK; ++n) {
-                o[t][n] *= alpha;
-                o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[n], pb, o[t][n], 0, 0, 0);
+                const bf16x8 v = __builtin_shufflevector(va[n][0], va[n][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb, o[t][n], 0, 0, 0);
             }
         }
     }
@@ -355,26 +370,36 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
     }
 }
 
-// merges the splits of mfma_decode_kernel.  grid = (tokens, q heads), 64 threads.
+// merges the splits of mfma_decode_kernel.  grid = (tokens, q heads), one wavefront each;
+// lane k holds (m, l) of split k (nsplit <= 64).  `mixed` != 0: the batch also holds
+// requests of the prefill kernel, whose tokens are left alone.
 __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __restrict__ ws_o,
                                                                 const float* __restrict__ ws_ml,
                                                                 const int32_t* __restrict__ cu_tokens,
                                                                 const int32_t* __restrict__ token_seq,
                                                                 bf16_t* __restrict__ out, int nq, int nkv, int D,
-                                                                int nsplit) {
+                                                                int nsplit, int mixed) {
     const int64_t tok = blockIdx.x;
     const int h = blockIdx.y;
-    const int s = token_seq[tok];
-    if ((cu_tokens[s + 1] - cu_tokens[s]) * (nq / nkv) > 16) return;
+    if (mixed) {
+        const int s = token_seq[tok];
+        if ((cu_tokens[s + 1] - cu_tokens[s]) * (nq / nkv) > 16) return;
+    }
+    const int lane = threadIdx.x;
     const int64_t head_row = tok * nq + h;
-    const float* ml = ws_ml + head_row * nsplit * 2;
-    float big = NEG_BIG;
-    for (int k = 0; k < nsplit; ++k) big = fmaxf(big, ml[2 * k]);
-    float den = 0.f;
-    for (int k = 0; k < nsplit; ++k) den += ml[2 * k + 1] * exp2f(ml[2 * k] - big);
-    for (int e = threadIdx.x; e < D; e += blockDim.x) {
+    float m = NEG_BIG, l = 0.f;
+    if (lane < nsplit) {
+        const float2 ml = *(const float2*)(ws_ml + (head_row * nsplit + lane) * 2);
+        m = ml.x;
+        l = ml.y;
+    }
+    const float big = wave_max(m);
+    const float f = exp2f(m - big);  // 0 for lanes without a split (l = 0 there anyway)
+    const float den = wave_sum(l * f);
+    const float* o = ws_o + head_row * nsplit * D;
+    for (int e = lane; e < D; e += LLE_WAVE) {
         float num = 0.f;
-        for (int k = 0; k < nsplit; ++k) num += ws_o[(head_row * nsplit + k) * D + e] * exp2f(ml[2 * k] - big);
+        for (int k = 0; k < nsplit; ++k) num += o[(int64_t)k * D + e] * __shfl(f, k, LLE_WAVE);
         out[head_row * D + e] = (bf16_t)(num / den);
     }
 }
@@ -383,7 +408,7 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 // each wavefront owns 32 rows and walks all keys up to its last row's position.
 #define PRE_RT 2
 template <int DK>
-__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_prefill_kernel(
+__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, 2) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, int nq, int nkv, int P, int64_t page_stride,
@@ -397,7 +422,8 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_prefill_kernel(
     if (nrows <= 16) return;  // the decode kernel's
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int row0 = (blockIdx.x * ATT_WAVES + wave) * (16 * PRE_RT);
+    // the last rows see the most keys: they are started first
+    const int row0 = ((gridDim.x - 1 - blockIdx.x) * ATT_WAVES + wave) * (16 * PRE_RT);
     if (row0 >= nrows) return;
     const int kv_len = kv_lens[s];
     const int past = kv_len - q_len;
@@ -452,7 +478,7 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
             max_pages, window, scale_log2);
         if (nsplit > 1)
             mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(ws_o, ws_ml, cu_tokens, token_seq, out, nq, nkv,
-                                                                      D, nsplit);
+                                                                      D, nsplit, run_prefill);
     }
     if (run_prefill) {
         const int rows = max_q_len * G;

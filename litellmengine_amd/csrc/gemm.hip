@@ -99,91 +99,113 @@ extern "C" int lle_gemm_nt_simt(const void* A, const void* B, void* C, int M, in
 typedef bf16_t gbf16x8 __attribute__((ext_vector_type(8)));
 typedef float gf32x4 __attribute__((ext_vector_type(4)));
 
-#define SK_WAVES 8
 #define SK_KSTEP 64
 
-template <int MT, typename TC>
+template <int MT, int NT, typename TC, int SK_WAVES, int UNROLL>
 __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                          const bf16_t* __restrict__ W,
                                                                          TC* __restrict__ C, int M, int N, int K) {
-    __shared__ float s_acc[SK_WAVES][MT][16][17];
+    // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
+    __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
-    const int64_t wrow = min(n0 + r16, (int64_t)N - 1);
-    const bf16_t* wp = W + wrow * K + 16 * c;
+    const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);
+    const bf16_t* wp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wp[nt] = W + min(n0 + 16 * nt + r16, (int64_t)N - 1) * K + 16 * c;
+    // rows of X beyond M are never written back, so their lanes may read any valid row
     const bf16_t* xp[MT];
-    bool xok[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = 16 * mt + r16;
-        xok[mt] = m < M;
-        xp[mt] = X + (int64_t)(xok[mt] ? m : 0) * K + 16 * c;
-    }
-    gf32x4 acc[MT];
+    for (int mt = 0; mt < MT; ++mt) xp[mt] = X + (int64_t)min(16 * mt + r16, M - 1) * K + 16 * c;
+    gf32x4 acc[NT][MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
     const gbf16x8 zero = {(bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f,
                           (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f, (bf16_t)0.f};
 
     const int full_steps = K / SK_KSTEP;
     int ss = wave;
-#pragma unroll 4
-    for (; ss < full_steps; ss += SK_WAVES) {
-        const int k0 = ss * SK_KSTEP;
-        const gbf16x8 w0 = *(const gbf16x8*)(wp + k0);
-        const gbf16x8 w1 = *(const gbf16x8*)(wp + k0 + 8);
+    // UNROLL steps at a time: all their loads are issued before the first product
+    for (; ss + (UNROLL - 1) * SK_WAVES < full_steps; ss += UNROLL * SK_WAVES) {
+        gbf16x8 w0[UNROLL][NT], w1[UNROLL][NT], x0[UNROLL][MT], x1[UNROLL][MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            gbf16x8 x0 = zero, x1 = zero;
-            if (xok[mt]) {
-                x0 = *(const gbf16x8*)(xp[mt] + k0);
-                x1 = *(const gbf16x8*)(xp[mt] + k0 + 8);
+        for (int u = 0; u < UNROLL; ++u) {
+            const int k0 = (ss + u * SK_WAVES) * SK_KSTEP;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                w0[u][nt] = *(const gbf16x8*)(wp[nt] + k0);
+                w1[u][nt] = *(const gbf16x8*)(wp[nt] + k0 + 8);
             }
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[mt], 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                x0[u][mt] = *(const gbf16x8*)(xp[mt] + k0);
+                x1[u][mt] = *(const gbf16x8*)(xp[mt] + k0 + 8);
+            }
         }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[u][nt], x0[u][mt], acc[nt][mt], 0, 0, 0);
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[u][nt], x1[u][mt], acc[nt][mt], 0, 0, 0);
+                }
     }
-    // the tail of K (a multiple of 8): one more step, taken by the wavefront whose turn it is
-    if (full_steps * SK_KSTEP < K && ss == full_steps) {
-        const int k0 = full_steps * SK_KSTEP;
+    // what is left of K: single steps; the last one may be partial (K is a multiple of 8),
+    // and there both operands are zeroed beyond K so that nothing outside the matrices is read
+    const int all_steps = (K + SK_KSTEP - 1) / SK_KSTEP;
+    for (; ss < all_steps; ss += SK_WAVES) {
+        const int k0 = ss * SK_KSTEP;
         const bool in0 = k0 + 16 * c + 8 <= K, in1 = k0 + 16 * c + 16 <= K;
-        const gbf16x8 w0 = in0 ? *(const gbf16x8*)(wp + k0) : zero;
-        const gbf16x8 w1 = in1 ? *(const gbf16x8*)(wp + k0 + 8) : zero;
+        gbf16x8 x0[MT], x1[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            const gbf16x8 x0 = (in0 && xok[mt]) ? *(const gbf16x8*)(xp[mt] + k0) : zero;
-            const gbf16x8 x1 = (in1 && xok[mt]) ? *(const gbf16x8*)(xp[mt] + k0 + 8) : zero;
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[mt], 0, 0, 0);
+            x0[mt] = in0 ? *(const gbf16x8*)(xp[mt] + k0) : zero;
+            x1[mt] = in1 ? *(const gbf16x8*)(xp[mt] + k0 + 8) : zero;
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            const gbf16x8 w0 = in0 ? *(const gbf16x8*)(wp[nt] + k0) : zero;
+            const gbf16x8 w1 = in1 ? *(const gbf16x8*)(wp[nt] + k0 + 8) : zero;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0[mt], acc[nt][mt], 0, 0, 0);
+                acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1[mt], acc[nt][mt], 0, 0, 0);
+            }
         }
     }
     // lane holds C^T[n = 4c + i][m = r16]
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_acc[wave][mt][4 * c + i][r16] = acc[mt][i];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_acc[wave][nt][mt][4 * c + i][r16] = acc[nt][mt][i];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
-        const int mt = idx / 256, m = (idx / 16) % 16, n = idx % 16;
-        const int64_t row = 16 * mt + m, col = n0 + n;
+    for (int idx = threadIdx.x; idx < NT * MT * 256; idx += blockDim.x) {
+        const int nt = idx / (MT * 256), mt = (idx / 256) % MT, m = (idx / 16) % 16, n = idx % 16;
+        const int64_t row = 16 * mt + m, col = n0 + 16 * nt + n;
         if (row >= M || col >= N) continue;
         float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][mt][n][m];
+        for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][nt][mt][n][m];
         C[row * N + col] = from_f32<TC>(sum);
     }
 }
 
-template <typename TC>
+template <typename TC, int NT>
 static int launch_skinny(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K, hipStream_t stream) {
-    const int blocks = (N + 15) / 16;
+    constexpr int WAVES = 16, UNROLL = 4 / NT;
+    const int blocks = (N + 16 * NT - 1) / (16 * NT);
     const int mt = (M + 15) / 16;
     switch (mt) {
-        case 1: gemm_skinny_kernel<1, TC><<<blocks, SK_WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 2: gemm_skinny_kernel<2, TC><<<blocks, SK_WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 3: gemm_skinny_kernel<3, TC><<<blocks, SK_WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 4: gemm_skinny_kernel<4, TC><<<blocks, SK_WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 1: gemm_skinny_kernel<1, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 2: gemm_skinny_kernel<2, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 3: gemm_skinny_kernel<3, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 4: gemm_skinny_kernel<4, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();
@@ -194,8 +216,11 @@ extern "C" int lle_gemm_skinny_bf16(const void* X, const void* W, void* C, int M
                                     hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 8 != 0 || K <= 0) return (int)hipErrorInvalidValue;
-    if (out_dtype == LLE_F32) return launch_skinny<float>((const bf16_t*)X, (const bf16_t*)W, (float*)C, M, N, K, stream);
-    if (out_dtype == LLE_BF16)
-        return launch_skinny<bf16_t>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, stream);
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)W;
+    // one tile of W rows per workgroup measured best up to 16 rows of X (two tiles share the X
+    // operands but halve the number of workgroups; they only pay off from 16 rows on)
+    if (out_dtype == LLE_F32) return launch_skinny<float, 1>(x, w, (float*)C, M, N, K, stream);
+    if (out_dtype == LLE_BF16) return launch_skinny<bf16_t, 1>(x, w, (bf16_t*)C, M, N, K, stream);
     return (int)hipErrorInvalidValue;
 }

@@ -124,16 +124,20 @@ class HipOps:
     # -- matrix products -------------------------------------------------------
     def linear(self, x, weight, out_dtype=None) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
-        kernel (a true 32-bit product).  bfloat16 operands: up to SKINNY_MAX_ROWS rows
-        the weight-streaming matrix-core kernel (either result type); more rows go to
-        the library product (bfloat16 result) or the 32-bit-accumulate kernel."""
+        kernel (a true 32-bit product).  bfloat16 operands: few rows take the
+        weight-streaming matrix-core kernel (either result type, up to 64 rows for a
+        float32 result); more rows go to the library product (bfloat16 result) or the
+        32-bit-accumulate kernel (float32 result)."""
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape
         N = weight.shape[0]
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
         out_dtype = out_dtype or x.dtype
-        if x.dtype == torch.bfloat16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0 and not self.force_library_gemm:
+        skinny = x.dtype == torch.bfloat16 and K % 8 == 0 and not self.force_library_gemm and (
+            M <= self.SKINNY_MAX_ROWS or (out_dtype == torch.float32 and M <= 64)
+            or (M <= 16 and N * K <= self.SKINNY_SMALL_WEIGHT))
+        if skinny:
             out = torch.empty((M, N), dtype=out_dtype, device=x.device)
             self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
                       _ptr(x), _ptr(weight), _ptr(out), M, N, K, dtype_code(out_dtype))
@@ -145,7 +149,10 @@ class HipOps:
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
 
-    SKINNY_MAX_ROWS = 16  # up to here the weight-streaming kernel; above, the library product
+    # measured on MI355X: the weight-streaming kernel wins up to 8 rows for every weight, up to 16
+    # rows for weights of up to 32 Mi elements; above, the library product
+    SKINNY_MAX_ROWS = 8
+    SKINNY_SMALL_WEIGHT = 1 << 25
     force_library_gemm = False
 
     # -- attention ---------------------------------------------------------------
@@ -237,8 +244,10 @@ class HipOps:
         return out
 
     force_generic_attention = False  # tests flip this to compare the two families of kernels
-    DECODE_TARGET_BLOCKS = 1024
-    DECODE_MIN_STEPS_PER_SPLIT = 4  # one 32-key step per wavefront
+    # measured on MI355X: about one workgroup per CU and at least 16 32-key steps (four per
+    # wavefront) per split are best; more splits cost more in partial results than they gain
+    DECODE_TARGET_BLOCKS = 256
+    DECODE_MIN_STEPS_PER_SPLIT = 16
 
     def decode_splits(self, num_seqs: int, num_kv_heads: int, max_kv_len: int, window: int) -> int:
         """Key splits of the decode kernel: enough workgroups to fill the chip, but
