@@ -101,7 +101,9 @@ typedef float gf32x4 __attribute__((ext_vector_type(4)));
 
 #define SK_KSTEP 64
 
-template <int MT, int NT, typename TC, int SK_WAVES, int UNROLL>
+// GATED: W holds gate rows [0, N/2) and then up rows [N/2, N); a workgroup takes 16 gate rows
+// and the 16 up rows that go with them (NT = 2) and writes silu(gate) * up, C is [M, N/2].
+template <int MT, int NT, bool GATED, typename TC, int SK_WAVES, int UNROLL>
 __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                          const bf16_t* __restrict__ W,
                                                                          TC* __restrict__ C, int M, int N, int K) {
@@ -109,10 +111,14 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int64_t n0 = (int64_t)blockIdx.x * (16 * NT);
+    const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
     const bf16_t* wp[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) wp[nt] = W + min(n0 + 16 * nt + r16, (int64_t)N - 1) * K + 16 * c;
+    for (int nt = 0; nt < NT; ++nt) {
+        const int64_t wrow = GATED ? min(n0 + r16, (int64_t)N / 2 - 1) + nt * ((int64_t)N / 2)
+                                   : min(n0 + 16 * nt + r16, (int64_t)N - 1);
+        wp[nt] = W + wrow * K + 16 * c;
+    }
     // rows of X beyond M are never written back, so their lanes may read any valid row
     const bf16_t* xp[MT];
 #pragma unroll
@@ -185,6 +191,21 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
 #pragma unroll
             for (int i = 0; i < 4; ++i) s_acc[wave][nt][mt][4 * c + i][r16] = acc[nt][mt][i];
     __syncthreads();
+    if (GATED) {
+        for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
+            const int mt = idx / 256, m = (idx / 16) % 16, n = idx % 16;
+            const int64_t row = 16 * mt + m, col = n0 + n;
+            if (row >= M || col >= N / 2) continue;
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int w = 0; w < SK_WAVES; ++w) {
+                g += s_acc[w][0][mt][n][m];
+                u += s_acc[w][NT - 1][mt][n][m];
+            }
+            C[row * (N / 2) + col] = from_f32<TC>(g / (1.0f + expf(-g)) * u);
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < NT * MT * 256; idx += blockDim.x) {
         const int nt = idx / (MT * 256), mt = (idx / 256) % MT, m = (idx / 16) % 16, n = idx % 16;
         const int64_t row = 16 * mt + m, col = n0 + 16 * nt + n;
@@ -196,16 +217,18 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
     }
 }
 
-template <typename TC, int NT>
+template <typename TC, int NT, bool GATED>
 static int launch_skinny(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K, hipStream_t stream) {
     constexpr int WAVES = 16, UNROLL = 4 / NT;
-    const int blocks = (N + 16 * NT - 1) / (16 * NT);
+    const int rows = GATED ? N / 2 : N;
+    const int per_block = GATED ? 16 : 16 * NT;
+    const int blocks = (rows + per_block - 1) / per_block;
     const int mt = (M + 15) / 16;
     switch (mt) {
-        case 1: gemm_skinny_kernel<1, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 2: gemm_skinny_kernel<2, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 3: gemm_skinny_kernel<3, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 4: gemm_skinny_kernel<4, NT, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 1: gemm_skinny_kernel<1, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 2: gemm_skinny_kernel<2, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 3: gemm_skinny_kernel<3, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 4: gemm_skinny_kernel<4, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();
@@ -220,7 +243,16 @@ extern "C" int lle_gemm_skinny_bf16(const void* X, const void* W, void* C, int M
     const bf16_t* w = (const bf16_t*)W;
     // one tile of W rows per workgroup measured best up to 16 rows of X (two tiles share the X
     // operands but halve the number of workgroups; they only pay off from 16 rows on)
-    if (out_dtype == LLE_F32) return launch_skinny<float, 1>(x, w, (float*)C, M, N, K, stream);
-    if (out_dtype == LLE_BF16) return launch_skinny<bf16_t, 1>(x, w, (bf16_t*)C, M, N, K, stream);
+    if (out_dtype == LLE_F32) return launch_skinny<float, 1, false>(x, w, (float*)C, M, N, K, stream);
+    if (out_dtype == LLE_BF16) return launch_skinny<bf16_t, 1, false>(x, w, (bf16_t*)C, M, N, K, stream);
     return (int)hipErrorInvalidValue;
+}
+
+// The gated feed-forward's first half in one launch: W [2I, K] holds the gate rows and then the
+// up rows; C [M, I] = silu(X gate^T) * (X up^T), the activation in 32-bit.  1 <= M <= 32.
+extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C, int M, int N2, int K,
+                                          hipStream_t stream) {
+    if (M <= 0 || N2 <= 0) return 0;
+    if (M > 32 || K % 8 != 0 || K <= 0 || N2 % 2 != 0) return (int)hipErrorInvalidValue;
+    return launch_skinny<bf16_t, 2, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, stream);
 }

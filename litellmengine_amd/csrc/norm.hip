@@ -37,10 +37,88 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_kernel(float* __restrict__ h
     }
 }
 
+// four consecutive elements of either type as 32-bit floats
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+    static __device__ __forceinline__ float4 load(const float* p) { return *(const float4*)p; }
+    static __device__ __forceinline__ void store(float* p, float4 v) { *(float4*)p = v; }
+};
+template <> struct Quad<bf16_t> {
+    typedef bf16_t vec __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ float4 load(const bf16_t* p) {
+        const vec v = *(const vec*)p;
+        return make_float4((float)v[0], (float)v[1], (float)v[2], (float)v[3]);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, float4 v) {
+        *(vec*)p = vec{(bf16_t)v.x, (bf16_t)v.y, (bf16_t)v.z, (bf16_t)v.w};
+    }
+};
+
+__device__ __forceinline__ float4 load_weight4(const void* w, int i, int dtype) {
+    return dtype == LLE_F32 ? Quad<float>::load((const float*)w + i) : Quad<bf16_t>::load((const bf16_t*)w + i);
+}
+
+// The same sums in one pass for rows of up to 256 * 4 * NORM_CHUNKS elements (a multiple of 4):
+// every thread keeps its part of the row in registers between the sum and the scaling.
+#define NORM_CHUNKS 8
+template <typename T>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ hidden, const T* __restrict__ delta,
+                                                              const int32_t* __restrict__ rows,
+                                                              const void* __restrict__ weight, int weight_dtype,
+                                                              T* __restrict__ out, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    const int64_t row = rows ? (int64_t)rows[r] : r;
+    float* h = hidden + row * H;
+    const T* dl = delta ? delta + row * H : nullptr;
+    float4 v[NORM_CHUNKS];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NORM_CHUNKS; ++k) {
+        const int i = (k * 256 + threadIdx.x) * 4;
+        if (i < H) {
+            float4 x = *(const float4*)(h + i);
+            if (dl) {
+                const float4 d = Quad<T>::load(dl + i);
+                x.x += d.x;
+                x.y += d.y;
+                x.z += d.z;
+                x.w += d.w;
+                if (!rows) *(float4*)(h + i) = x;
+            }
+            v[k] = x;
+            ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        }
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    T* o = out + r * H;
+#pragma unroll
+    for (int k = 0; k < NORM_CHUNKS; ++k) {
+        const int i = (k * 256 + threadIdx.x) * 4;
+        if (i < H) {
+            const float4 w = load_weight4(weight, i, weight_dtype);
+            Quad<T>::store(o + i, make_float4(v[k].x * inv * w.x, v[k].y * inv * w.y, v[k].z * inv * w.z,
+                                              v[k].w * inv * w.w));
+        }
+    }
+}
+
 extern "C" int lle_add_rmsnorm(void* hidden, const void* delta, const void* rows, const void* weight,
                                int weight_dtype, void* out, int R, int H, float eps, int dtype,
                                hipStream_t stream) {
     if (R <= 0) return 0;
+    if (H % 4 == 0 && H <= 256 * 4 * NORM_CHUNKS) {
+        if (dtype == LLE_F32)
+            add_rmsnorm_vec_kernel<float><<<R, 256, 0, stream>>>((float*)hidden, (const float*)delta,
+                                                                  (const int32_t*)rows, weight, weight_dtype,
+                                                                  (float*)out, H, eps);
+        else
+            add_rmsnorm_vec_kernel<bf16_t><<<R, 256, 0, stream>>>((float*)hidden, (const bf16_t*)delta,
+                                                                   (const int32_t*)rows, weight, weight_dtype,
+                                                                   (bf16_t*)out, H, eps);
+        LLE_RETURN_LAUNCH_STATUS();
+    }
     int threads = 256;
     if (H > 2048) threads = 512;
     if (H > 8192) threads = 1024;

@@ -269,13 +269,33 @@ class HipOps:
                   _ptr(gate_up), _ptr(out), N, two_i // 2, dtype_code(gate_up.dtype))
         return out
 
+    def gate_up_silu(self, x, weight) -> torch.Tensor:
+        """x [M, K], weight [2 I, K] (gate rows, then up rows) -> silu(x gate^T) * (x up^T), [M, I].
+        Few bfloat16 rows run as ONE weight-streaming launch with the activation in its
+        epilogue; otherwise the product and silu_mul."""
+        _dev(x, "x")
+        _dev(weight, "weight", x.dtype)
+        M, K = x.shape
+        N2 = weight.shape[0]
+        _need(weight.shape[1] == K and N2 % 2 == 0, f"weight {list(weight.shape)} does not fit x [{M}, {K}]")
+        if (x.dtype == torch.bfloat16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0 and not self.force_library_gemm):
+            out = torch.empty((M, N2 // 2), dtype=x.dtype, device=x.device)
+            self._run("gemm", "lle_gemm_skinny_gated_bf16", [_P, _P, _P, _I, _I, _I, _P],
+                      _ptr(x), _ptr(weight), _ptr(out), M, N2, K)
+            return out
+        return self.silu_mul(self.linear(x, weight))
+
     # -- picking tokens --------------------------------------------------------------
     def argmax(self, logits) -> torch.Tensor:
         """float32 [R, V] -> int32 [R], first maximum wins."""
         _dev(logits, "logits", torch.float32)
         R, V = logits.shape
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
-        self._run("sampling", "lle_argmax_rows", [_P, _P, _I, _I, _P], _ptr(logits), _ptr(out), R, V)
+        chunks = max(1, min(64, V // 2048))  # enough workgroups to stream a long row from all CUs
+        part_val = torch.empty((R * chunks,), dtype=torch.float32, device=logits.device)
+        part_idx = torch.empty((R * chunks,), dtype=torch.int32, device=logits.device)
+        self._run("sampling", "lle_argmax_rows", [_P, _P, _P, _P, _I, _I, _I, _P],
+                  _ptr(logits), _ptr(out), _ptr(part_val), _ptr(part_idx), R, V, chunks)
         return out
 
     def sample(self, logits, temperature, uniform) -> torch.Tensor:

@@ -7,21 +7,11 @@ LLE_DEFINE_ERROR_STRING()
 
 #define SAMPLE_THREADS 1024
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void argmax_rows_kernel(const float* __restrict__ logits,
-                                                                     int32_t* __restrict__ out, int V) {
-    __shared__ float s_val[SAMPLE_THREADS / LLE_WAVE];
-    __shared__ int s_idx[SAMPLE_THREADS / LLE_WAVE];
-    const float* row = logits + (int64_t)blockIdx.x * V;
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best || best_i == 0x7fffffff) {  // strided ascending: first maximum of this thread
-            best = v;
-            best_i = i;
-        }
-    }
-    // a NaN never wins a ">" comparison; ties go to the smaller index
+#define ARGMAX_THREADS 256
+
+// (value, index) of the first maximum among the candidates of one workgroup; a NaN never
+// wins a ">" comparison; ties go to the smaller index.  Valid in thread 0.
+__device__ __forceinline__ void block_argmax(float& best, int& best_i, float* s_val, int* s_idx) {
     for (int o = LLE_WAVE / 2; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, LLE_WAVE);
         const int oi = __shfl_xor(best_i, o, LLE_WAVE);
@@ -37,18 +27,70 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void argmax_rows_kernel(const float
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < SAMPLE_THREADS / LLE_WAVE; ++w)
+        const int nwaves = (blockDim.x + LLE_WAVE - 1) / LLE_WAVE;
+        for (int w = 1; w < nwaves; ++w)
             if (s_val[w] > best || (s_val[w] == best && s_idx[w] < best_i)) {
                 best = s_val[w];
                 best_i = s_idx[w];
             }
-        out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
     }
 }
 
-extern "C" int lle_argmax_rows(const void* logits, void* out, int R, int V, hipStream_t stream) {
+// stage 1: grid (rows, chunks): the first maximum of one chunk of a row
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_chunks_kernel(const float* __restrict__ logits,
+                                                                        float* __restrict__ part_val,
+                                                                        int32_t* __restrict__ part_idx, int V) {
+    __shared__ float s_val[ARGMAX_THREADS / LLE_WAVE];
+    __shared__ int s_idx[ARGMAX_THREADS / LLE_WAVE];
+    const float* row = logits + (int64_t)blockIdx.x * V;
+    const int chunks = gridDim.y;
+    const int per = (V + chunks - 1) / chunks;
+    const int lo = min(V, (int)blockIdx.y * per), hi = min(V, lo + per);
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const float v = row[i];
+        if (v > best || best_i == 0x7fffffff) {  // ascending: the first maximum of this thread
+            best = v;
+            best_i = i;
+        }
+    }
+    block_argmax(best, best_i, s_val, s_idx);
+    if (threadIdx.x == 0) {
+        part_val[blockIdx.x * chunks + blockIdx.y] = best;
+        part_idx[blockIdx.x * chunks + blockIdx.y] = best_i;
+    }
+}
+
+// stage 2: grid rows, one wavefront: the first maximum among the chunks' winners
+__global__ __launch_bounds__(LLE_WAVE) void argmax_final_kernel(const float* __restrict__ part_val,
+                                                                const int32_t* __restrict__ part_idx,
+                                                                int32_t* __restrict__ out, int chunks) {
+    __shared__ float s_val[1];
+    __shared__ int s_idx[1];
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int k = threadIdx.x; k < chunks; k += blockDim.x) {
+        const float v = part_val[blockIdx.x * chunks + k];
+        const int i = part_idx[blockIdx.x * chunks + k];
+        if (i != 0x7fffffff && (v > best || best_i == 0x7fffffff || (v == best && i < best_i))) {
+            best = v;
+            best_i = i;
+        }
+    }
+    block_argmax(best, best_i, s_val, s_idx);
+    if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+// `part_val`, `part_idx`: workspaces of R * chunks elements
+extern "C" int lle_argmax_rows(const void* logits, void* out, void* part_val, void* part_idx, int R, int V,
+                               int chunks, hipStream_t stream) {
     if (R <= 0) return 0;
-    argmax_rows_kernel<<<R, SAMPLE_THREADS, 0, stream>>>((const float*)logits, (int32_t*)out, V);
+    if (chunks <= 0 || chunks > 65535) return (int)hipErrorInvalidValue;
+    argmax_chunks_kernel<<<dim3(R, chunks), ARGMAX_THREADS, 0, stream>>>((const float*)logits, (float*)part_val,
+                                                                          (int32_t*)part_idx, V);
+    argmax_final_kernel<<<R, LLE_WAVE, 0, stream>>>((const float*)part_val, (const int32_t*)part_idx, (int32_t*)out,
+                                                     chunks);
     LLE_RETURN_LAUNCH_STATUS();
 }
 

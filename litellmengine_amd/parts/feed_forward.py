@@ -28,4 +28,4 @@ class GatedMLP(FeedForward):
         self.down.bind(weights, ctx)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down.forward(self.ctx.ops.silu_mul(self.gate_up.forward(x)))
+        return self.down.forward(self.ctx.ops.gate_up_silu(x, self.gate_up.weight))

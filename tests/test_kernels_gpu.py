@@ -85,6 +85,19 @@ def test_silu_mul(dtype, I):
     assert (got.double() - want.double()).abs().max() < tol(dtype, 4)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,I,K", [(1, 128, 64), (5, 200, 96), (8, 12288, 4096), (8, 136, 80), (9, 100, 72), (40, 64, 48)])
+def test_gate_up_silu(dtype, M, I, K):
+    x = rnd((M, K), dtype, 21, 2.0)
+    w = rnd((2 * I, K), dtype, 22, 0.1)
+    got = ops().gate_up_silu(x, w)
+    gu = x.double() @ w.double().t()
+    want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+    assert got.shape == (M, I)
+    lim = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (got.double() - want).abs().max() < lim * max(1.0, want.abs().max().item())
+
+
 def test_silu_mul_reference_vector():
     # tests/test_silu_and_mul.cpp:48-56
     g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])

@@ -114,6 +114,9 @@ class TorchOps:
         g, u = gate_up[:, :I].to(self.cd), gate_up[:, I:].to(self.cd)
         return (g / (1.0 + torch.exp(-g)) * u).to(gate_up.dtype)
 
+    def gate_up_silu(self, x, weight):
+        return self.silu_mul(self.linear(x, weight))
+
     def argmax(self, logits):
         return torch.argmax(logits, dim=-1).to(torch.int32)  # torch returns the first maximum
 
