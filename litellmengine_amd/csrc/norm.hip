@@ -71,8 +71,13 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     const int64_t row = rows ? (int64_t)rows[r] : r;
     float* h = hidden + row * H;
     const T* dl = delta ? delta + row * H : nullptr;
-    float4 v[NORM_CHUNKS];
+    float4 v[NORM_CHUNKS], wv[NORM_CHUNKS];
     float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NORM_CHUNKS; ++k) {  // the weights do not wait for the sum
+        const int i = (k * 256 + threadIdx.x) * 4;
+        if (i < H) wv[k] = load_weight4(weight, i, weight_dtype);
+    }
 #pragma unroll
     for (int k = 0; k < NORM_CHUNKS; ++k) {
         const int i = (k * 256 + threadIdx.x) * 4;
@@ -97,7 +102,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     for (int k = 0; k < NORM_CHUNKS; ++k) {
         const int i = (k * 256 + threadIdx.x) * 4;
         if (i < H) {
-            const float4 w = load_weight4(weight, i, weight_dtype);
+            const float4 w = wv[k];
             Quad<T>::store(o + i, make_float4(v[k].x * inv * w.x, v[k].y * inv * w.y, v[k].z * inv * w.z,
                                               v[k].w * inv * w.w));
         }
