@@ -83,3 +83,54 @@ def test_graph_replays_equal_eager_steps(tmp_path, dtype):
     assert (outs[True] - outs[False]).abs().max() < TOL[dtype] / 4
     want = plain.model_logits_fast(seqs[0], w, cfg)
     assert (outs[True][0].double() - want[20]).abs().max() < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(tmp_path, dtype):
+    """A short prompt, then hundreds of tokens one by one (several pages, several
+    context buckets of the decode graphs); the very first positions of a sequence
+    (position 0 sees itself only) are checked on their own."""
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(600, cfg["vocab_size"], 77)
+    want = plain.model_logits_fast(tokens, w, cfg)
+    runner = make_runner(d, dtype, 16, 40)
+    slot = runner.admit()
+    first = runner.step([StepEntry(slot, tokens[:1], [0])]).cpu()
+    assert (first.double() - want[:1]).abs().max() < TOL[dtype]
+    second = runner.step([StepEntry(slot, tokens[1:3], [0, 1])]).cpu()
+    assert (second.double() - want[1:3]).abs().max() < TOL[dtype]
+    worst = 0.0
+    for i in range(3, 600):
+        got = runner.step([StepEntry(slot, [tokens[i]], [0])], borrow=True)
+        if i % 7 == 0 or i > 590:
+            worst = max(worst, (got.cpu().double() - want[i : i + 1]).abs().max().item())
+    assert worst < TOL[dtype], worst
+    runner.release(slot)
+
+
+def test_qwen3_8b_layer_sizes(tmp_path):
+    """Two layers at the Qwen3-8B layer sizes (hidden 4096, 32/8 heads of 128, feed-forward
+    12288, vocabulary 151936): float32 against the plain implementation in three cuttings,
+    bfloat16 against the same."""
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.weights import write_model_dir
+
+    cfg = Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_size=4096, num_attention_heads=32,
+        num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1e6,
+        rms_norm_eps=1e-6, tie_word_embeddings=False))
+    d = str(tmp_path / "m8b")
+    write_model_dir(cfg, d, 3, torch.bfloat16)
+    pcfg, w = plain.read_model_dir(d, dtype=torch.float32)
+    tokens = random_tokens(70, cfg.vocab_size, 5)
+    want = plain.model_logits_fast(tokens, w, pcfg).double()
+    scale = max(1.0, want.abs().max().item())
+    for dtype, tol in (("float32", 2e-4), ("bfloat16", 4e-2)):  # the oracle itself is float32 here
+        runner = make_runner(d, dtype, 16, 8)
+        for cuts in ([70], [38] + [1] * 32, [2, 17, 3, 30, 18]):
+            got = run_cut(runner, tokens, cuts)
+            err = (got.double() - want).abs().max().item() / scale
+            assert err < tol, (dtype, cuts, err)
+        del runner
+        torch.cuda.empty_cache()
