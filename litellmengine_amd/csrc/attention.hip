@@ -24,7 +24,8 @@
 //    per group; the four wavefronts take every fourth 32-key step; partial
 //    (m, l, acc) of the splits are merged by the combine kernel.
 //  * mfma_prefill_kernel: same tile code, 32 rows (token, head) per wavefront,
-//    all keys up to each row's own position.
+//    all keys up to each row's own position; the four wavefronts of a workgroup
+//    share the K/V tiles through LDS.
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -154,46 +155,131 @@ struct RowInfo {
 // leaves registers, and the softmax state of row r sits in the lanes r + 16c.
 // The k slots of the second product are (tile A keys 4c..4c+3, tile B keys 4c..4c+3).
 template <int DK, int RT>
-__device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16_t* __restrict__ kv_layer,
-                                            const int32_t* __restrict__ table, int kvh, int nkv, int P,
-                                            int64_t page_stride, int step_begin, int step_end, int step_stride,
-                                            int lo_min, int hi, float scale_log2, f32x4 (&o)[RT][2 * DK],
-                                            float (&m)[RT], float (&l)[RT]) {
-    constexpr int D = DK * 32;
-    const int lane = threadIdx.x % LLE_WAVE;
-    const int c = lane / 16, r16 = lane % 16;
-
-    bf16x8 qv[RT][DK];
+struct RowState {
+    bf16x8 qv[RT][DK];             // Q^T operands of the lane's row
     int open_lo[RT], open_hi[RT];  // steps with open_lo <= j0 and j0 + 31 <= open_hi need no mask
+    f32x4 o[RT][2 * DK];           // O^T tiles: value elements 16 n + 4 c .. + 3 of row r16
+    float m[RT], l[RT];            // running maximum (base 2) and this lane's share of the sum
+};
+
+template <int DK, int RT>
+__device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT]) {
+    const int c = (threadIdx.x % LLE_WAVE) / 16;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks) {
             if (row[t].q) {
-                qv[t][ks] = *(const bf16x8*)(row[t].q + 32 * ks + 8 * c);
+                st.qv[t][ks] = *(const bf16x8*)(row[t].q + 32 * ks + 8 * c);
             } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qv[t][ks][i] = (bf16_t)0.0f;
+                for (int i = 0; i < 8; ++i) st.qv[t][ks][i] = (bf16_t)0.0f;
             }
         }
 #pragma unroll
-        for (int n = 0; n < 2 * DK; ++n) o[t][n] = f32x4{0.f, 0.f, 0.f, 0.f};
-        m[t] = NEG_BIG;
-        l[t] = 0.f;
+        for (int n = 0; n < 2 * DK; ++n) st.o[t][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+        st.m[t] = NEG_BIG;
+        st.l[t] = 0.f;
         int lo_max = row[t].q ? row[t].lo : 0, pos_min = row[t].q ? row[t].pos : 0x7fffffff;
 #pragma unroll
         for (int off = 1; off < LLE_WAVE; off <<= 1) {
             lo_max = max(lo_max, __shfl_xor(lo_max, off, LLE_WAVE));
             pos_min = min(pos_min, __shfl_xor(pos_min, off, LLE_WAVE));
         }
-        open_lo[t] = lo_max;
-        open_hi[t] = pos_min == 0x7fffffff ? -1 : pos_min;
+        st.open_lo[t] = lo_max;
+        st.open_hi[t] = pos_min == 0x7fffffff ? -1 : pos_min;
     }
+}
+
+// One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key r16 of
+// half-tile x, elements 32 ks + 8 c .. + 7.  load_v(n): value element 16 n + r16, keys 4c..4c+3
+// of half-tile 0 then of half-tile 1.  Each operand is fetched once and used by all row tiles.
+template <int DK, int RT, typename LoadK, typename LoadV>
+__device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&row)[RT], LoadK load_k,
+                                          LoadV load_v, int j0, float scale_log2) {
+    const int c = (threadIdx.x % LLE_WAVE) / 16;
+    f32x4 s[RT][2];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) s[t][0] = s[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) {
+            const bf16x8 k = load_k(x, ks);
+#pragma unroll
+            for (int t = 0; t < RT; ++t)
+                s[t][x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k, st.qv[t][ks], s[t][x], 0, 0, 0);
+        }
+    bf16x8 pb[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        // scores of row r16 for keys j0 + 16 x + 4 c + i, in the base-2 domain
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sc[i] = s[t][i / 4][i % 4] * scale_log2;
+        if (!(j0 >= st.open_lo[t] && j0 + KSTEP - 1 <= st.open_hi[t])) {  // same for the whole wavefront
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int j = j0 + 16 * (i / 4) + 4 * c + (i % 4);
+                if (j < row[t].lo || j > row[t].pos) sc[i] = NEG_BIG;
+            }
+        }
+        float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                               fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
+        const float new_m = fmaxf(st.m[t], tile_max);
+        // a masked score is NEG_BIG; while the row has seen no key yet new_m is NEG_BIG too,
+        // and exp2(0) = 1 would count the masked key: shift such rows so that they give 0
+        const float base = new_m <= NEG_BIG ? 0.f : new_m;
+        const float alpha = __builtin_amdgcn_exp2f(st.m[t] - base);
+        st.m[t] = new_m;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float p = __builtin_amdgcn_exp2f(sc[i] - base);
+            psum += p;
+            pb[t][i] = (bf16_t)p;
+        }
+        st.l[t] = st.l[t] * alpha + psum;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum moved somewhere
+#pragma unroll
+            for (int n = 0; n < 2 * DK; ++n) st.o[t][n] *= alpha;
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < 2 * DK; ++n) {
+        const bf16x8 v = load_v(n);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) st.o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[t], st.o[t][n], 0, 0, 0);
+    }
+}
+
+// the partial sums of a row sit in the four lanes r16 + 16 c
+template <int DK, int RT>
+__device__ __forceinline__ void finish_rows(RowState<DK, RT>& st) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+        st.l[t] += __shfl_xor(st.l[t], 16, LLE_WAVE);
+        st.l[t] += __shfl_xor(st.l[t], 32, LLE_WAVE);
+    }
+}
+
+// The steps step_begin, step_begin + step_stride, ... < step_end with the operands loaded by
+// each wavefront straight from the pages.
+template <int DK, int RT>
+__device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT],
+                                            const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ table,
+                                            int kvh, int nkv, int P, int64_t page_stride, int step_begin,
+                                            int step_end, int step_stride, int lo_min, int hi, float scale_log2) {
+    constexpr int D = DK * 32;
+    const int lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    init_rows<DK, RT>(st, row);
     const int64_t k_head = (int64_t)kvh * P * D;
     const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
-
-    for (int st = step_begin; st < step_end; st += step_stride) {
-        const int j0 = st * KSTEP;
+    for (int step = step_begin; step < step_end; step += step_stride) {
+        const int j0 = step * KSTEP;
         const bf16_t* page[2];
         int off[2];
 #pragma unroll
@@ -204,77 +290,23 @@ __device__ __forceinline__ void attend_rows(const RowInfo (&row)[RT], const bf16
             page[x] = kv_layer + (int64_t)table[probe / P] * page_stride;
             off[x] = jx % P;
         }
-        // K operands: lane (c, r16) holds key r16 of the tile, elements 32 ks + 8 c .. + 7
         bf16x8 ka[2][DK];
 #pragma unroll
         for (int x = 0; x < 2; ++x)
 #pragma unroll
             for (int ks = 0; ks < DK; ++ks)
                 ka[x][ks] = *(const bf16x8*)(page[x] + k_head + (int64_t)(off[x] + r16) * D + 32 * ks + 8 * c);
-        // V^T operands: lane holds value element 16 n + r16, keys 4c..4c+3 of tile A then of tile B
         bf16x4 va[2 * DK][2];
 #pragma unroll
         for (int n = 0; n < 2 * DK; ++n)
 #pragma unroll
             for (int x = 0; x < 2; ++x)
                 va[n][x] = *(const bf16x4*)(page[x] + v_head + (int64_t)(16 * n + r16) * P + off[x] + 4 * c);
-#pragma unroll
-        for (int t = 0; t < RT; ++t) {
-            f32x4 s[2];
-#pragma unroll
-            for (int x = 0; x < 2; ++x) {
-                s[x] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int ks = 0; ks < DK; ++ks)
-                    s[x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[x][ks], qv[t][ks], s[x], 0, 0, 0);
-            }
-            // scores of row r16 for keys j0 + 16 x + 4 c + i, in the base-2 domain
-            float sc[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sc[i] = s[i / 4][i % 4] * scale_log2;
-            if (!(j0 >= open_lo[t] && j0 + KSTEP - 1 <= open_hi[t])) {  // same for the whole wavefront
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int j = j0 + 16 * (i / 4) + 4 * c + (i % 4);
-                    if (j < row[t].lo || j > row[t].pos) sc[i] = NEG_BIG;
-                }
-            }
-            float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                   fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
-            const float new_m = fmaxf(m[t], tile_max);
-            // a masked score is NEG_BIG; while the row has seen no key yet new_m is NEG_BIG too,
-            // and exp2(0) = 1 would count the masked key: shift such rows so that they give 0
-            const float base = new_m <= NEG_BIG ? 0.f : new_m;
-            const float alpha = __builtin_amdgcn_exp2f(m[t] - base);
-            m[t] = new_m;
-            float psum = 0.f;
-            bf16x8 pb;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float p = __builtin_amdgcn_exp2f(sc[i] - base);
-                psum += p;
-                pb[i] = (bf16_t)p;
-            }
-            l[t] = l[t] * alpha + psum;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum moved somewhere
-#pragma unroll
-                for (int n = 0; n < 2 * DK; ++n) o[t][n] *= alpha;
-            }
-#pragma unroll
-            for (int n = 0; n < 2 * DK; ++n) {
-                const bf16x8 v = __builtin_shufflevector(va[n][0], va[n][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb, o[t][n], 0, 0, 0);
-            }
-        }
+        tile_step<DK, RT>(
+            st, row, [&](int x, int ks) { return ka[x][ks]; },
+            [&](int n) { return __builtin_shufflevector(va[n][0], va[n][1], 0, 1, 2, 3, 4, 5, 6, 7); }, j0, scale_log2);
     }
-    // the partial sums of a row sit in the four lanes r16 + 16 c
-#pragma unroll
-    for (int t = 0; t < RT; ++t) {
-        l[t] += __shfl_xor(l[t], 16, LLE_WAVE);
-        l[t] += __shfl_xor(l[t], 32, LLE_WAVE);
-    }
+    finish_rows<DK, RT>(st);
 }
 
 // row `r` of the (token, head-in-group) rows of one request and kv head
@@ -329,19 +361,18 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int sb = first + split * per_split;
     const int se = min(last + 1, sb + per_split);
 
-    f32x4 o[1][2 * DK];
-    float m[1], l[1];
-    attend_rows<DK, 1>(row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, ATT_WAVES, lo_min, hi,
-                       scale_log2, o, m, l);
+    RowState<DK, 1> st;
+    attend_rows<DK, 1>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, ATT_WAVES, lo_min, hi,
+                       scale_log2);
 
     // merge the four wavefronts
 #pragma unroll
     for (int n = 0; n < 2 * DK; ++n)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_o[(wave * 16 + r16) * D + 16 * n + 4 * c + i] = o[0][n][i];
+        for (int i = 0; i < 4; ++i) s_o[(wave * 16 + r16) * D + 16 * n + 4 * c + i] = st.o[0][n][i];
     if (c == 0) {
-        s_m[wave * 16 + r16] = m[0];
-        s_l[wave * 16 + r16] = l[0];
+        s_m[wave * 16 + r16] = st.m[0];
+        s_l[wave * 16 + r16] = st.l[0];
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
@@ -404,55 +435,147 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     }
 }
 
-// Requests with more than 16 rows.  grid = (row blocks of 128, kv heads, requests);
-// each wavefront owns 32 rows and walks all keys up to its last row's position.
-#define PRE_RT 2
+// Requests with more than 16 rows.  grid = (row blocks of 128, kv heads, requests); each
+// wavefront owns 32 rows.  The 32-key tiles of K and V^T are copied from the pages into LDS
+// once per workgroup (all 256 threads, the next tile while this one is multiplied) and every
+// wavefront reads its matrix-core operands from there: 128 rows share one pass over the keys.
+//   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
+//   LDS V^T tile: [D][32 keys + 4]
+// row tiles per wavefront: two while the accumulators fit the register file
+#define PRE_RT_OF(DK) ((DK) <= 4 ? 2 : 1)
 template <int DK>
-__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, 2) void mfma_prefill_kernel(
+__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, int nq, int nkv, int P, int64_t page_stride,
     int max_pages, int window, float scale_log2) {
     constexpr int D = DK * 32;
+    constexpr int PRE_RT = PRE_RT_OF(DK);
+    constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT;
+    constexpr int KROW = D + 8;       // elements per key row in LDS
+    constexpr int VROW = KSTEP + 4;   // elements per value-element row in LDS
+    constexpr int TILE = KSTEP * KROW + D * VROW;
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * TILE];
+
     const int s = blockIdx.z, kvh = blockIdx.y;
     const int G = nq / nkv;
     const int q_start = cu_tokens[s];
     const int q_len = cu_tokens[s + 1] - q_start;
     const int nrows = q_len * G;
     if (nrows <= 16) return;  // the decode kernel's
+    // the last rows see the most keys: they are started first
+    const int block_row0 = (gridDim.x - 1 - blockIdx.x) * PRE_ROWS;
+    if (block_row0 >= nrows) return;
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    // the last rows see the most keys: they are started first
-    const int row0 = ((gridDim.x - 1 - blockIdx.x) * ATT_WAVES + wave) * (16 * PRE_RT);
-    if (row0 >= nrows) return;
     const int kv_len = kv_lens[s];
     const int past = kv_len - q_len;
     const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
 
+    // the workgroup's key range, and this wavefront's own
+    const int block_last_row = min(nrows, block_row0 + PRE_ROWS) - 1;
+    const int hi = past + block_last_row / G;
+    const int block_first_pos = past + block_row0 / G;
+    const int lo_min = window > 0 ? max(0, block_first_pos - window + 1) : 0;
+    const int first_step = lo_min / KSTEP, end_step = hi / KSTEP + 1;
+
+    const int row0 = block_row0 + wave * (16 * PRE_RT);
     RowInfo row[PRE_RT];
 #pragma unroll
     for (int t = 0; t < PRE_RT; ++t) row[t] = make_row(q, row0 + 16 * t + r16, nrows, G, q_start, past, nq, kvh, D, window);
-    const int first_pos = past + row0 / G;
-    const int last_row = min(nrows, row0 + 16 * PRE_RT) - 1;
-    const int hi = past + last_row / G;
-    const int lo_min = window > 0 ? max(0, first_pos - window + 1) : 0;
+    int my_first = end_step, my_end = first_step;  // a wavefront without rows multiplies nothing
+    if (row0 < nrows) {
+        const int my_last_row = min(nrows, row0 + 16 * PRE_RT) - 1;
+        const int my_lo = window > 0 ? max(0, past + row0 / G - window + 1) : 0;
+        my_first = my_lo / KSTEP;
+        my_end = (past + my_last_row / G) / KSTEP + 1;
+    }
+    RowState<DK, PRE_RT> st;
+    init_rows<DK, PRE_RT>(st, row);
 
-    f32x4 o[PRE_RT][2 * DK];
-    float m[PRE_RT], l[PRE_RT];
-    attend_rows<DK, PRE_RT>(row, kv_layer, table, kvh, nkv, P, page_stride, lo_min / KSTEP, hi / KSTEP + 1, 1,
-                            lo_min, hi, scale_log2, o, m, l);
+    const int64_t k_head = (int64_t)kvh * P * D;
+    const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
+    // a tile holds 4 D 16-byte pieces of K and as many of V^T; this thread copies NP of each
+    constexpr int PIECES = 4 * D;
+    constexpr int NP = (PIECES + ATT_WAVES * LLE_WAVE - 1) / (ATT_WAVES * LLE_WAVE);
+    bf16x8 stage_k[NP], stage_v[NP];
+    auto fetch = [&](int step) {
+        const int j0 = step * KSTEP;
+        const bf16_t* page[2];
+        int off[2];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            const int jx = j0 + 16 * x;
+            const int probe = min(max(jx, lo_min), hi);
+            page[x] = kv_layer + (int64_t)table[probe / P] * page_stride;
+            off[x] = jx % P;
+        }
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int piece = threadIdx.x + ATT_WAVES * LLE_WAVE * i;
+            if (piece < PIECES) {
+                const int key = piece / (D / 8), ch = piece % (D / 8);  // key 0..31, 16-byte piece of its row
+                const int xk = key / 16;
+                stage_k[i] = *(const bf16x8*)((xk ? page[1] : page[0]) + k_head +
+                                              (int64_t)((xk ? off[1] : off[0]) + key % 16) * D + ch * 8);
+                const int dd = piece / 4, part = piece % 4;  // value element 0..D-1, quarter of its 32 keys
+                const int xv = part / 2;
+                stage_v[i] = *(const bf16x8*)((xv ? page[1] : page[0]) + v_head + (int64_t)dd * P +
+                                              (xv ? off[1] : off[0]) + (part % 2) * 8);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+        bf16_t* kt = lds + buf * TILE;
+        bf16_t* vt = kt + KSTEP * KROW;
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int piece = threadIdx.x + ATT_WAVES * LLE_WAVE * i;
+            if (piece < PIECES) {
+                const int key = piece / (D / 8), ch = piece % (D / 8);
+                *(bf16x8*)(kt + key * KROW + ch * 8) = stage_k[i];
+                const int dd = piece / 4, part = piece % 4;
+                bf16_t* dst = vt + dd * VROW + (part / 2) * 16 + (part % 2) * 8;  // 8-byte aligned
+                *(bf16x4*)dst = __builtin_shufflevector(stage_v[i], stage_v[i], 0, 1, 2, 3);
+                *(bf16x4*)(dst + 4) = __builtin_shufflevector(stage_v[i], stage_v[i], 4, 5, 6, 7);
+            }
+        }
+    };
+
+    fetch(first_step);
+    stash(0);
+    __syncthreads();
+    for (int step = first_step; step < end_step; ++step) {
+        const int buf = (step - first_step) & 1;
+        const bool more = step + 1 < end_step;
+        if (more) fetch(step + 1);
+        if (step >= my_first && step < my_end) {
+            const bf16_t* kt = lds + buf * TILE;
+            const bf16_t* vt = kt + KSTEP * KROW;
+            tile_step<DK, PRE_RT>(
+                st, row, [&](int x, int ks) { return *(const bf16x8*)(kt + (16 * x + r16) * KROW + 32 * ks + 8 * c); },
+                [&](int n) {
+                    const bf16_t* p = vt + (16 * n + r16) * VROW + 4 * c;
+                    return __builtin_shufflevector(*(const bf16x4*)p, *(const bf16x4*)(p + 16), 0, 1, 2, 3, 4, 5, 6, 7);
+                },
+                step * KSTEP, scale_log2);
+        }
+        if (more) stash(buf ^ 1);
+        __syncthreads();
+    }
+    finish_rows<DK, PRE_RT>(st);
 #pragma unroll
     for (int t = 0; t < PRE_RT; ++t) {
         const int r = row0 + 16 * t + r16;
         if (r >= nrows) continue;
         const int tk = r / G, g = r - tk * G;
         bf16_t* dst = out + ((int64_t)(q_start + tk) * nq + kvh * G + g) * D;
-        const float inv = 1.0f / l[t];
+        const float inv = 1.0f / st.l[t];
 #pragma unroll
         for (int n = 0; n < 2 * DK; ++n) {
             bf16x4 v;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(o[t][n][i] * inv);
+            for (int i = 0; i < 4; ++i) v[i] = (bf16_t)(st.o[t][n][i] * inv);
             *(bf16x4*)(dst + 16 * n + 4 * c) = v;
         }
     }
@@ -482,7 +605,8 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
     }
     if (run_prefill) {
         const int rows = max_q_len * G;
-        const int blocks = (rows + ATT_WAVES * 16 * PRE_RT - 1) / (ATT_WAVES * 16 * PRE_RT);
+        constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT_OF(DK);
+        const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
         mfma_prefill_kernel<DK><<<dim3(blocks, nkv, S), ATT_WAVES * LLE_WAVE, 0, stream>>>(
             q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, nq, nkv, P, page_stride, max_pages, window,
             scale_log2);

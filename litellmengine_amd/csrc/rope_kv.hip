@@ -84,12 +84,110 @@ __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
     }
 }
 
+// The same for bfloat16 heads of 16, 32, 64, 128 or 256 elements with a rotation over a
+// multiple of 16 elements (or none): a lane holds 8 consecutive elements (16-byte loads and
+// stores), d / 8 lanes hold a head, a wavefront holds 512 / d heads of one token.  The partner of
+// element i in the rotation is i +- rot / 2, which lies rot / 16 lanes away.
+typedef bf16_t rbf16x8 __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
+    const bf16_t* __restrict__ qkv, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+    const void* __restrict__ q_weight, const void* __restrict__ k_weight, int weight_dtype,
+    const float* __restrict__ inv_freq, int rot, float eps, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kv_layer,
+    int nq, int nkv, int d, int page_size, int64_t page_stride, int write_kv, int total_heads) {
+    const int lph = d / 8;  // lanes per head
+    const int lane = threadIdx.x % LLE_WAVE;
+    const int heads_per_wave = LLE_WAVE / lph;
+    const int64_t gw = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LLE_WAVE;  // global wavefront
+    const int64_t flat = gw * heads_per_wave + lane / lph;                           // (token, head)
+    const int hl = lane % lph;                                                        // lane inside the head
+    const int per_token = nq + 2 * nkv;
+    const bool live = flat < (int64_t)total_heads;
+    const int64_t n = live ? flat / per_token : 0;
+    const int head = live ? (int)(flat - n * per_token) : 0;
+    const bool is_q = head < nq;
+    const bool is_k = !is_q && head < nq + nkv;
+    const int e0 = 8 * hl;
+
+    float x[8];
+    {
+        const rbf16x8 v = *(const rbf16x8*)(qkv + (n * per_token + head) * d + e0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = (float)v[i];
+    }
+    if (is_q || is_k) {
+        const void* w = is_q ? q_weight : k_weight;
+        if (w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+            for (int o = 1; o < lph; o <<= 1) ss += __shfl_xor(ss, o, LLE_WAVE);
+            const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = x[i] * inv * load_as_f32(w, e0 + i, weight_dtype);
+        }
+        if (rot > 0) {
+            const int half = rot / 2;
+            const int dl = half / 8;  // lanes between partners
+            const bool low = e0 < half, in_rot = e0 < rot;
+            const float pos = (float)positions[n];
+            float other[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                // lanes of the low half read from lane + dl, those of the high half from lane - dl
+                const float up = __shfl_down(x[i], dl, LLE_WAVE), down = __shfl_up(x[i], dl, LLE_WAVE);
+                other[i] = low ? up : down;
+            }
+            if (in_rot) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int fi = (low ? e0 : e0 - half) + i;
+                    float sn, cs;
+                    sincosf(pos * inv_freq[fi], &sn, &cs);
+                    x[i] = low ? x[i] * cs - other[i] * sn : x[i] * cs + other[i] * sn;
+                }
+            }
+        }
+    }
+    if (!live) return;
+    rbf16x8 y;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = (bf16_t)x[i];
+    if (is_q) {
+        *(rbf16x8*)(q_out + (n * nq + head) * d + e0) = y;
+        return;
+    }
+    if (!write_kv) return;
+    const int slot = slots[n];
+    if (slot < 0) return;
+    const int64_t page = slot / page_size;
+    const int off = slot - (int)page * page_size;
+    bf16_t* page_base = kv_layer + page * page_stride;
+    if (is_k) {
+        *(rbf16x8*)(page_base + ((int64_t)(head - nq) * page_size + off) * d + e0) = y;
+    } else {
+        bf16_t* v = page_base + ((int64_t)nkv + (head - nq - nkv)) * page_size * d + off;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[(int64_t)(e0 + i) * page_size] = y[i];
+    }
+}
+
 extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* positions, const void* slots,
                                       const void* q_weight, const void* k_weight, int weight_dtype,
                                       const void* inv_freq, int rot, float eps, void* q_out, void* kv_layer,
                                       int N, int nq, int nkv, int d, int page_size, int64_t page_stride,
                                       int write_kv, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
+    const bool pow2 = d == 16 || d == 32 || d == 64 || d == 128 || d == 256;
+    if (dtype == LLE_BF16 && pow2 && rot % 16 == 0 && (int64_t)N * (nq + 2 * nkv) < (1ll << 31)) {
+        const int total_heads = N * (nq + 2 * nkv);
+        const int heads_per_block = 4 * (LLE_WAVE / (d / 8));
+        const int blocks = (total_heads + heads_per_block - 1) / heads_per_block;
+        qk_norm_rope_write_vec_kernel<<<blocks, 256, 0, stream>>>(
+            (const bf16_t*)qkv, (const int32_t*)positions, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
+            (const float*)inv_freq, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
+            write_kv, total_heads);
+        LLE_RETURN_LAUNCH_STATUS();
+    }
     dim3 grid(N, nq + 2 * nkv);
     if (dtype == LLE_F32)
         qk_norm_rope_write_kernel<float><<<grid, 64, 0, stream>>>(

@@ -137,7 +137,8 @@ def make_cache(num_pages, nkv, P, d, dtype, seed):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,d,P,rot,norm", [(4, 2, 16, 4, 16, True), (6, 3, 48, 3, 48, True),
                                                  (8, 1, 128, 16, 128, True), (2, 2, 80, 8, 32, False),
-                                                 (3, 1, 256, 5, 0, True)])
+                                                 (3, 1, 256, 5, 0, True), (4, 2, 64, 16, 32, True),
+                                                 (5, 5, 32, 8, 32, False), (32, 8, 128, 16, 128, True)])
 def test_qk_norm_rope_write(dtype, nq, nkv, d, P, rot, norm):
     N, pages = 9, 6
     qkv = rnd((N, (nq + 2 * nkv) * d), dtype, 8)
