@@ -328,8 +328,11 @@ __device__ __forceinline__ RowInfo make_row(const bf16_t* q, int r, int nrows, i
 
 // Requests whose rows (q_len * group) fit one 16-row tile: decoded tokens and very
 // short portions.  grid = (requests, kv heads, splits).
+#ifndef DEC_WAVES
+#define DEC_WAVES 4
+#endif
 template <int DK>
-__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
+__global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
@@ -338,8 +341,8 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
     constexpr int D = DK * 32;
     extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
     float* s_o = smem;
-    float* s_m = smem + ATT_WAVES * 16 * D;
-    float* s_l = s_m + ATT_WAVES * 16;
+    float* s_m = smem + DEC_WAVES * 16 * D;
+    float* s_l = s_m + DEC_WAVES * 16;
 
     const int s = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, nsplit = gridDim.z;
     const int G = nq / nkv;
@@ -362,14 +365,14 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int se = min(last + 1, sb + per_split);
 
     RowState<DK, 1> st;
-    attend_rows<DK, 1>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, ATT_WAVES, lo_min, hi,
+    attend_rows<DK, 1>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi,
                        scale_log2);
 
-    // merge the four wavefronts
+    // merge the wavefronts (rows that do not exist are not worth the LDS traffic)
+    if (r16 < nrows) {
 #pragma unroll
-    for (int n = 0; n < 2 * DK; ++n)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s_o[(wave * 16 + r16) * D + 16 * n + 4 * c + i] = st.o[0][n][i];
+        for (int n = 0; n < 2 * DK; ++n) *(f32x4*)(s_o + (wave * 16 + r16) * D + 16 * n + 4 * c) = st.o[0][n];
+    }
     if (c == 0) {
         s_m[wave * 16 + r16] = st.m[0];
         s_l[wave * 16 + r16] = st.l[0];
@@ -379,10 +382,10 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void mfma_decode_kernel(
         const int r = idx / D, e = idx - r * D;
         float big = s_m[r];
 #pragma unroll
-        for (int w = 1; w < ATT_WAVES; ++w) big = fmaxf(big, s_m[w * 16 + r]);
+        for (int w = 1; w < DEC_WAVES; ++w) big = fmaxf(big, s_m[w * 16 + r]);
         float num = 0.f, den = 0.f;
 #pragma unroll
-        for (int w = 0; w < ATT_WAVES; ++w) {
+        for (int w = 0; w < DEC_WAVES; ++w) {
             const float f = exp2f(s_m[w * 16 + r] - big);
             num += s_o[(w * 16 + r) * D + e] * f;
             den += s_l[w * 16 + r] * f;
@@ -590,13 +593,13 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
     constexpr int D = DK * 32;
     const int G = nq / nkv;
     if (run_decode) {
-        const size_t smem = (size_t)(ATT_WAVES * 16 * D + 2 * ATT_WAVES * 16) * sizeof(float);
+        const size_t smem = (size_t)(DEC_WAVES * 16 * D + 2 * DEC_WAVES * 16) * sizeof(float);
         if (smem > 64 * 1024) {
             hipError_t e = hipFuncSetAttribute((const void*)mfma_decode_kernel<DK>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e != hipSuccess) return (int)e;
         }
-        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit), ATT_WAVES * LLE_WAVE, smem, stream>>>(
+        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit), DEC_WAVES * LLE_WAVE, smem, stream>>>(
             q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, nq, nkv, P, page_stride,
             max_pages, window, scale_log2);
         if (nsplit > 1)
