@@ -156,19 +156,29 @@ class HipOps:
     force_library_gemm = False
 
     # -- attention ---------------------------------------------------------------
-    def qk_norm_rope_write(self, qkv, positions, slots, q_weight, k_weight, inv_freq, rotary_dim: int,
-                           eps: float, kv_layer, num_q_heads: int, num_kv_heads: int, head_dim: int,
-                           write_kv: bool = True) -> torch.Tensor:
-        """qkv [N, (nq + 2 nkv) d] -> q [N, nq, d] normed and rotated; K (normed, rotated)
-        and V go to the pages `kv_layer` [pages, 2, nkv, page_size, d] at `slots` [N]."""
-        _dev(qkv, "qkv")
+    def rope_table(self, positions, inv_freq) -> torch.Tensor:
+        """cos and sin of float(position) * inv_freq for every token: float32 [N, len(inv_freq), 2].
+        Made once per step; every head of every layer with this rotation reads it."""
         _dev(positions, "positions", torch.int32)
+        _dev(inv_freq, "inv_freq", torch.float32)
+        N, half = positions.shape[0], inv_freq.shape[0]
+        out = torch.empty((N, half, 2), dtype=torch.float32, device=positions.device)
+        self._run("rope_kv", "lle_rope_table", [_P, _P, _P, _I, _I, _P], _ptr(positions), _ptr(inv_freq), _ptr(out),
+                  N, half)
+        return out
+
+    def qk_norm_rope_write(self, qkv, slots, q_weight, k_weight, cos_sin, rotary_dim: int, eps: float, kv_layer,
+                           num_q_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True) -> torch.Tensor:
+        """qkv [N, (nq + 2 nkv) d] -> q [N, nq, d] normed and rotated; K (normed, rotated)
+        and V go to the pages `kv_layer` [pages, 2, nkv, page_size, d] at `slots` [N].
+        `cos_sin` is rope_table()'s [N, rotary_dim / 2, 2] (None when rotary_dim is 0)."""
+        _dev(qkv, "qkv")
         _dev(slots, "slots", torch.int32)
         _dev(kv_layer, "kv_layer", qkv.dtype)
         nq, nkv, d = num_q_heads, num_kv_heads, head_dim
         N = qkv.shape[0]
         _need(qkv.shape == (N, (nq + 2 * nkv) * d), "qkv has the wrong width")
-        _need(positions.shape == (N,) and slots.shape == (N,), "positions and slots must be [N]")
+        _need(slots.shape == (N,), "slots must be [N]")
         _need(kv_layer.dim() == 5 and kv_layer.shape[1] == 2 and kv_layer.shape[2] == nkv
               and kv_layer.shape[4] == d, "kv_layer must be [pages, 2, nkv, page_size, d]")
         _need(0 <= rotary_dim <= d and rotary_dim % 2 == 0, "rotary_dim must be even and <= head_dim")
@@ -181,14 +191,14 @@ class HipOps:
         if q_weight is not None and k_weight is not None:
             _need(q_weight.dtype == k_weight.dtype, "q_norm and k_norm weights must share a type")
         if rotary_dim > 0:
-            _dev(inv_freq, "inv_freq", torch.float32)
-            _need(inv_freq.shape == (rotary_dim // 2,), "inv_freq must be [rotary_dim / 2]")
+            _dev(cos_sin, "cos_sin", torch.float32)
+            _need(cos_sin.shape == (N, rotary_dim // 2, 2), "cos_sin must be [N, rotary_dim / 2, 2]")
         page_size = kv_layer.shape[3]
         q_out = torch.empty((N, nq, d), dtype=qkv.dtype, device=qkv.device)
         self._run("rope_kv", "lle_qk_norm_rope_write",
-                  [_P, _P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _P],
-                  _ptr(qkv), _ptr(positions), _ptr(slots), _ptr(q_weight), _ptr(k_weight), wd,
-                  _ptr(inv_freq) if rotary_dim > 0 else None, rotary_dim, float(eps), _ptr(q_out), _ptr(kv_layer),
+                  [_P, _P, _P, _P, _I, _P, _I, _F, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _P],
+                  _ptr(qkv), _ptr(slots), _ptr(q_weight), _ptr(k_weight), wd,
+                  _ptr(cos_sin) if rotary_dim > 0 else None, rotary_dim, float(eps), _ptr(q_out), _ptr(kv_layer),
                   N, nq, nkv, d, page_size, kv_layer.stride(0), 1 if write_kv else 0, dtype_code(qkv.dtype))
         return q_out
 

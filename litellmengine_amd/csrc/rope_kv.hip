@@ -9,7 +9,9 @@
 //   k head:  norm over d (weight [d]) -> rotate -> K page of the token's slot
 //   v head:  copy                               -> V page of the token's slot
 // Rotation pairs element i with i + rot/2 (half split) for i < rot/2; elements
-// >= rot pass through.  angle = float(pos) * inv_freq[i], all in 32-bit.
+// >= rot pass through.  angle = float(pos) * inv_freq[i], all in 32-bit; cosine and sine of
+// every (token, i) are computed once per step by rope_table_kernel ([N][rot/2][2] floats) and
+// shared by all heads and all layers.
 // A cache page holds K as [nkv][page_size][d] and then V as [nkv][d][page_size]
 // (V is kept transposed so that the matrix-core attention kernels find the keys
 // of one value column next to each other); slot = page * page_size + offset;
@@ -20,10 +22,10 @@ LLE_DEFINE_ERROR_STRING()
 
 template <typename T>
 __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
-    const T* __restrict__ qkv, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
-    const void* __restrict__ q_weight, const void* __restrict__ k_weight, int weight_dtype,
-    const float* __restrict__ inv_freq, int rot, float eps, T* __restrict__ q_out, T* __restrict__ kv_layer,
-    int nq, int nkv, int d, int page_size, int64_t page_stride, int write_kv) {
+    const T* __restrict__ qkv, const int32_t* __restrict__ slots, const void* __restrict__ q_weight,
+    const void* __restrict__ k_weight, int weight_dtype, const float* __restrict__ cos_sin, int rot, float eps,
+    T* __restrict__ q_out, T* __restrict__ kv_layer, int nq, int nkv, int d, int page_size, int64_t page_stride,
+    int write_kv) {
     const int64_t n = blockIdx.x;
     const int head = blockIdx.y;  // 0..nq-1 q, then nkv k, then nkv v
     const int lane = threadIdx.x;
@@ -63,7 +65,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
         inv = 1.0f / sqrtf(ss / (float)d + eps);
     }
     const int half = rot / 2;
-    const float pos = (float)positions[n];
+    const float2* cs = (const float2*)cos_sin + n * half;
     for (int i = lane; i < half; i += LLE_WAVE) {
         float x1 = to_f32<T>(src[i]) * inv;
         float x2 = to_f32<T>(src[i + half]) * inv;
@@ -71,9 +73,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
             x1 *= load_as_f32(w, i, weight_dtype);
             x2 *= load_as_f32(w, i + half, weight_dtype);
         }
-        const float ang = pos * inv_freq[i];
-        float s, c;
-        sincosf(ang, &s, &c);
+        const float c = cs[i].x, s = cs[i].y;
         dst[i] = from_f32<T>(x1 * c - x2 * s);
         dst[i + half] = from_f32<T>(x2 * c + x1 * s);
     }
@@ -90,10 +90,11 @@ __global__ __launch_bounds__(64) void qk_norm_rope_write_kernel(
 // element i in the rotation is i +- rot / 2, which lies rot / 16 lanes away.
 typedef bf16_t rbf16x8 __attribute__((ext_vector_type(8)));
 __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
-    const bf16_t* __restrict__ qkv, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
-    const void* __restrict__ q_weight, const void* __restrict__ k_weight, int weight_dtype,
-    const float* __restrict__ inv_freq, int rot, float eps, bf16_t* __restrict__ q_out, bf16_t* __restrict__ kv_layer,
-    int nq, int nkv, int d, int page_size, int64_t page_stride, int write_kv, int total_heads) {
+    const bf16_t* __restrict__ qkv, const int32_t* __restrict__ slots, const void* __restrict__ q_weight,
+    const void* __restrict__ k_weight, int weight_dtype, const float* __restrict__ cos_sin, int rot, float eps,
+    bf16_t* __restrict__ q_out, bf16_t* __restrict__ kv_layer, int nq, int nkv, int d, int page_size,
+    int64_t page_stride, int write_kv, int total_heads) {
+    // write_kv: 0 = q only, 1 = K and V, 2 = K only (another kernel writes V)
     const int lph = d / 8;  // lanes per head
     const int lane = threadIdx.x % LLE_WAVE;
     const int heads_per_wave = LLE_WAVE / lph;
@@ -129,7 +130,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
             const int half = rot / 2;
             const int dl = half / 8;  // lanes between partners
             const bool low = e0 < half, in_rot = e0 < rot;
-            const float pos = (float)positions[n];
             float other[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -138,12 +138,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
                 other[i] = low ? up : down;
             }
             if (in_rot) {
+                // 8 (cos, sin) pairs = four 16-byte loads
+                const float4* tab = (const float4*)(cos_sin + (n * half + (low ? e0 : e0 - half)) * 2);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int fi = (low ? e0 : e0 - half) + i;
-                    float sn, cs;
-                    sincosf(pos * inv_freq[fi], &sn, &cs);
-                    x[i] = low ? x[i] * cs - other[i] * sn : x[i] * cs + other[i] * sn;
+                for (int i = 0; i < 4; ++i) {
+                    const float4 t = tab[i];  // cos, sin of element 2i, then of 2i + 1
+                    x[2 * i] = low ? x[2 * i] * t.x - other[2 * i] * t.y : x[2 * i] * t.x + other[2 * i] * t.y;
+                    x[2 * i + 1] = low ? x[2 * i + 1] * t.z - other[2 * i + 1] * t.w
+                                       : x[2 * i + 1] * t.z + other[2 * i + 1] * t.w;
                 }
             }
         }
@@ -164,16 +166,89 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
     bf16_t* page_base = kv_layer + page * page_stride;
     if (is_k) {
         *(rbf16x8*)(page_base + ((int64_t)(head - nq) * page_size + off) * d + e0) = y;
-    } else {
+    } else if (write_kv == 1) {
         bf16_t* v = page_base + ((int64_t)nkv + (head - nq - nkv)) * page_size * d + off;
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[(int64_t)(e0 + i) * page_size] = y[i];
     }
 }
 
-extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* positions, const void* slots,
+// The V heads of many tokens into the transposed pages.  A workgroup takes 16 consecutive
+// tokens of the batch and one kv head: the rows are read whole into LDS, and every thread
+// writes one value element of 8 tokens, as one 16-byte store when those tokens sit in
+// consecutive slots of one page starting at a multiple of 8 (prompt portions do), else one by one.
+#define VW_TOKENS 16
+__global__ __launch_bounds__(256) void v_write_transposed_kernel(const bf16_t* __restrict__ qkv,
+                                                                  const int32_t* __restrict__ slots,
+                                                                  bf16_t* __restrict__ kv_layer, int N, int nq, int nkv,
+                                                                  int d, int page_size, int64_t page_stride) {
+    extern __shared__ bf16_t tile[];  // [VW_TOKENS][d + 2]
+    __shared__ int s_slot[VW_TOKENS];
+    const int t0 = blockIdx.x * VW_TOKENS, kvh = blockIdx.y;
+    const int width = (nq + 2 * nkv) * d;
+    const int row = d + 2;
+    for (int idx = threadIdx.x; idx < VW_TOKENS * (d / 8); idx += blockDim.x) {
+        const int t = idx / (d / 8), ch = idx % (d / 8);
+        if (t0 + t < N) {
+            const rbf16x8 v = *(const rbf16x8*)(qkv + (int64_t)(t0 + t) * width + (int64_t)(nq + nkv + kvh) * d + 8 * ch);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tile[t * row + 8 * ch + i] = v[i];
+        }
+    }
+    if (threadIdx.x < VW_TOKENS) s_slot[threadIdx.x] = t0 + threadIdx.x < N ? slots[t0 + threadIdx.x] : -1;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 2 * d; idx += blockDim.x) {
+        const int g = idx / d, e = idx - g * d;  // tokens 8 g .. 8 g + 7, value element e
+        const int first = s_slot[8 * g];
+        bool run = first >= 0 && first % 8 == 0 && first % page_size + 8 <= page_size;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) run = run && s_slot[8 * g + i] == first + i;
+        if (run) {
+            const int64_t page = first / page_size;
+            const int off = first - (int)page * page_size;
+            rbf16x8 y;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = tile[(8 * g + i) * row + e];
+            *(rbf16x8*)(kv_layer + page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off) = y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int slot = s_slot[8 * g + i];
+                if (slot < 0) continue;
+                const int64_t page = slot / page_size;
+                const int off = slot - (int)page * page_size;
+                kv_layer[page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off] =
+                    tile[(8 * g + i) * row + e];
+            }
+        }
+    }
+}
+
+// cos and sin of float(pos) * inv_freq[i] for every token of the step: out [N][half][2]
+__global__ __launch_bounds__(256) void rope_table_kernel(const int32_t* __restrict__ positions,
+                                                          const float* __restrict__ inv_freq,
+                                                          float* __restrict__ out, int64_t total, int half) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t n = idx / half;
+    const int i = (int)(idx - n * half);
+    float s, c;
+    sincosf((float)positions[n] * inv_freq[i], &s, &c);
+    ((float2*)out)[idx] = make_float2(c, s);
+}
+
+extern "C" int lle_rope_table(const void* positions, const void* inv_freq, void* out, int N, int half,
+                              hipStream_t stream) {
+    const int64_t total = (int64_t)N * half;
+    if (total <= 0) return 0;
+    rope_table_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>((const int32_t*)positions,
+                                                                      (const float*)inv_freq, (float*)out, total, half);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* slots,
                                       const void* q_weight, const void* k_weight, int weight_dtype,
-                                      const void* inv_freq, int rot, float eps, void* q_out, void* kv_layer,
+                                      const void* cos_sin, int rot, float eps, void* q_out, void* kv_layer,
                                       int N, int nq, int nkv, int d, int page_size, int64_t page_stride,
                                       int write_kv, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
@@ -182,22 +257,26 @@ extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* positions, co
         const int total_heads = N * (nq + 2 * nkv);
         const int heads_per_block = 4 * (LLE_WAVE / (d / 8));
         const int blocks = (total_heads + heads_per_block - 1) / heads_per_block;
+        // many tokens: V goes through the transposing kernel (16-byte stores into the pages)
+        const bool split_v = write_kv && N >= 64 && page_size % 8 == 0 && (N + VW_TOKENS - 1) / VW_TOKENS <= 0x7fffffff;
         qk_norm_rope_write_vec_kernel<<<blocks, 256, 0, stream>>>(
-            (const bf16_t*)qkv, (const int32_t*)positions, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
-            (const float*)inv_freq, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
-            write_kv, total_heads);
+            (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, rot, eps,
+            (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride, write_kv ? (split_v ? 2 : 1) : 0,
+            total_heads);
+        if (split_v)
+            v_write_transposed_kernel<<<dim3((N + VW_TOKENS - 1) / VW_TOKENS, nkv), 256,
+                                        VW_TOKENS * (d + 2) * sizeof(bf16_t), stream>>>(
+                (const bf16_t*)qkv, (const int32_t*)slots, (bf16_t*)kv_layer, N, nq, nkv, d, page_size, page_stride);
         LLE_RETURN_LAUNCH_STATUS();
     }
     dim3 grid(N, nq + 2 * nkv);
     if (dtype == LLE_F32)
         qk_norm_rope_write_kernel<float><<<grid, 64, 0, stream>>>(
-            (const float*)qkv, (const int32_t*)positions, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
-            (const float*)inv_freq, rot, eps, (float*)q_out, (float*)kv_layer, nq, nkv, d, page_size, page_stride,
-            write_kv);
+            (const float*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, rot, eps,
+            (float*)q_out, (float*)kv_layer, nq, nkv, d, page_size, page_stride, write_kv);
     else
         qk_norm_rope_write_kernel<bf16_t><<<grid, 64, 0, stream>>>(
-            (const bf16_t*)qkv, (const int32_t*)positions, (const int32_t*)slots, q_weight, k_weight, weight_dtype,
-            (const float*)inv_freq, rot, eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
-            write_kv);
+            (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, rot, eps,
+            (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride, write_kv);
     LLE_RETURN_LAUNCH_STATUS();
 }

@@ -48,6 +48,7 @@ class StepState:
     max_q_len: int
     max_kv_len: int  # host-side bounds; they choose kernels, never results
     seqs: Optional[List[SeqInfo]]  # the same on the host (None inside a captured graph)
+    scratch: dict = dataclasses.field(default_factory=dict)  # what parts make once per step and share
 
 
 @dataclasses.dataclass

@@ -103,6 +103,7 @@ class DecoderLM:
     def forward(self, step, caches) -> torch.Tensor:
         """Run the tokens of `step` (engine.batch.StepState) through the plan and
         return float32 logits [len(step.logit_rows), vocab]."""
+        step.scratch.clear()  # per-step tables are made anew in every run (also when a graph is captured)
         hidden = self.embedding.forward(step.token_ids)
         delta = None
         for i, e in enumerate(self.plan):

@@ -80,13 +80,13 @@ class PagedAttention(Mixer):
     def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
         ops = self.ctx.ops
         qkv = self.qkv.forward(x)
-        fused = self.position.fused_rotary()
+        fused = self.position.fused_rotary(step)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
         group = cache.group
         if fused is not None:
-            inv_freq, rot = fused
+            cos_sin, rot = fused
             q = ops.qk_norm_rope_write(
-                qkv, step.positions, group.slot_mapping, self.q_norm_w, self.k_norm_w, inv_freq, rot, eps,
+                qkv, group.slot_mapping, self.q_norm_w, self.k_norm_w, cos_sin, rot, eps,
                 cache.kv, self.nq, self.nkv, self.d, cache.writes,
             )
         else:
@@ -101,7 +101,7 @@ class PagedAttention(Mixer):
             q, k = self.position.apply(q.view(N, self.nq, self.d), k.view(N, self.nkv, self.d), step.positions)
             packed = torch.cat([q.reshape(N, qw), k.reshape(N, kw), qkv[:, qw + kw :]], dim=1).contiguous()
             q = ops.qk_norm_rope_write(
-                packed, step.positions, group.slot_mapping, None, None, None, 0, 0.0,
+                packed, group.slot_mapping, None, None, None, 0, 0.0,
                 cache.kv, self.nq, self.nkv, self.d, cache.writes,
             )
         a = ops.paged_attention(

@@ -66,12 +66,13 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Encodes positions into q and k.  `fused_rotary()` may return
-    (inv_freq float32 [rotary_dim / 2], rotary_dim) when the encoding is a
-    half-split rotation that the fused q/k kernel can apply itself; otherwise
-    `apply` is called on q [N, nq, d] and k [N, nkv, d] (it may work in place)."""
+    """Encodes positions into q and k.  `fused_rotary(step)` may return
+    (cos_sin float32 [N, rotary_dim / 2, 2], rotary_dim) when the encoding is a
+    half-split rotation that the fused q/k kernel can apply itself (`step.scratch`
+    is a dictionary that lives for one step: tables made once go there);
+    otherwise `apply` is called on q [N, nq, d] and k [N, nkv, d]."""
 
-    def fused_rotary(self):
+    def fused_rotary(self, step):
         return None
 
     def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor):

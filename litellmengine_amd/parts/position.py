@@ -15,7 +15,8 @@ class RotaryHalfSplit(PositionEncoding):
     (src/layers/rotary.cu:81-83, :96-116; the reference rotates the whole head,
     rot = head_dim, and computes angles on the fly with no table).  The
     frequencies are computed once in double precision and rounded to float32;
-    the angle, sine and cosine are float32 in the kernel."""
+    the angle, sine and cosine are float32 in the kernel, computed once per step for
+    all heads and layers."""
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: Optional[int] = None):
         self.head_dim = head_dim
@@ -31,12 +32,19 @@ class RotaryHalfSplit(PositionEncoding):
         inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -(2.0 * i) / self.rotary_dim)
         self.inv_freq = inv.to(torch.float32).to(ctx.device)
 
-    def fused_rotary(self):
-        return self.inv_freq, self.rotary_dim
+    def fused_rotary(self, step):
+        # cosines and sines of this step's positions: made by the first layer that asks,
+        # shared by every layer with the same rotation
+        key = ("rope_table", self.theta, self.rotary_dim)
+        table = step.scratch.get(key)
+        if table is None:
+            table = self.ctx.ops.rope_table(step.positions, self.inv_freq)
+            step.scratch[key] = table
+        return table, self.rotary_dim
 
 
 class NoPositionEncoding(PositionEncoding):
     """q and k pass unchanged (a mixer whose order comes from elsewhere)."""
 
-    def fused_rotary(self):
+    def fused_rotary(self, step):
         return None, 0

@@ -152,15 +152,45 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, P, rot, norm):
         inv = (1e6 ** (-(2.0 * i) / rot)).float().cuda()
     kv_got = make_cache(pages, nkv, P, d, dtype, 11)
     kv_ref = kv_got.clone()
-    q_got = ops().qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv_got, nq, nkv, d)
-    q_ref = REF.qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv_ref, nq, nkv, d)
+    cs = ops().rope_table(positions, inv) if rot else None
+    if rot:
+        assert (cs.double() - REF.rope_table(positions, inv).double()).abs().max() < 2e-6
+    q_got = ops().qk_norm_rope_write(qkv, slots, qw, kw, cs, rot, 1e-6, kv_got, nq, nkv, d)
+    q_ref = REF.qk_norm_rope_write(qkv, slots, qw, kw, REF.rope_table(positions, inv) if rot else None, rot, 1e-6,
+                                   kv_ref, nq, nkv, d)
     t = tol(dtype, 8)
     assert (q_got.double() - q_ref.double()).abs().max() < t
     assert (kv_got.double() - kv_ref.double()).abs().max() < t
     # a reader entry leaves the pages alone
     kv2 = kv_ref.clone()
-    ops().qk_norm_rope_write(qkv, positions, slots, qw, kw, inv, rot, 1e-6, kv2, nq, nkv, d, write_kv=False)
+    ops().qk_norm_rope_write(qkv, slots, qw, kw, cs, rot, 1e-6, kv2, nq, nkv, d, write_kv=False)
     assert torch.equal(kv2, kv_ref)
+
+
+@pytest.mark.parametrize("P", [8, 16, 64])
+def test_qk_norm_rope_write_many_tokens(P):
+    """Enough tokens for the transposing V writer: a prompt portion in consecutive slots that
+    starts in the middle of a page, single tokens elsewhere, and tokens that are not written."""
+    dtype, nq, nkv, d = torch.bfloat16, 8, 2, 128
+    pages = 40
+    end = 3 * P + 5 + 83
+    slots = list(range(3 * P + 5, end)) + [-1, 1, end + 3, -1, end + 2 * P - 1, 0, 2]
+    N = len(slots)
+    qkv = rnd((N, (nq + 2 * nkv) * d), dtype, 31)
+    positions = torch.arange(N, dtype=torch.int32).cuda() + 11
+    slots = torch.tensor(slots, dtype=torch.int32).cuda()
+    qw = (1 + 0.1 * rnd((d,), torch.float32, 32)).to(dtype)
+    kw = (1 + 0.1 * rnd((d,), torch.float32, 33)).to(dtype)
+    i = torch.arange(d // 2, dtype=torch.float64)
+    inv = (1e6 ** (-(2.0 * i) / d)).float().cuda()
+    kv_got = make_cache(pages, nkv, P, d, dtype, 34)
+    kv_ref = kv_got.clone()
+    cs = ops().rope_table(positions, inv)
+    q_got = ops().qk_norm_rope_write(qkv, slots, qw, kw, cs, d, 1e-6, kv_got, nq, nkv, d)
+    q_ref = REF.qk_norm_rope_write(qkv, slots, qw, kw, REF.rope_table(positions, inv), d, 1e-6, kv_ref, nq, nkv, d)
+    assert (q_got.double() - q_ref.double()).abs().max() < 0.1
+    assert (kv_got.double() - kv_ref.double()).abs().max() < 0.1
+    assert torch.equal(v_pages(kv_got), v_pages(kv_ref))  # values are copied, not computed
 
 
 def test_rotary_reference_vector():
@@ -172,7 +202,7 @@ def test_rotary_reference_vector():
     slots = torch.tensor([-1, -1], dtype=torch.int32).cuda()
     inv = torch.tensor([1.0, 1e4 ** -0.5]).cuda()
     kv = torch.zeros(1, 2, 1, 4, 4).cuda()
-    got = ops().qk_norm_rope_write(qkv, positions, slots, None, None, inv, 4, 0.0, kv, 2, 1, 4).cpu()
+    got = ops().qk_norm_rope_write(qkv, slots, None, None, ops().rope_table(positions, inv), 4, 0.0, kv, 2, 1, 4).cpu()
     assert torch.allclose(got[0].reshape(-1), q[0], atol=1e-7)
     x = q[1].reshape(2, 4)
     want = torch.empty(2, 4)

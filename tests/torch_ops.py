@@ -47,7 +47,11 @@ class TorchOps:
     def linear(self, x, weight, out_dtype=None):
         return (x.to(self.cd) @ weight.to(self.cd).t()).to(out_dtype or x.dtype)
 
-    def qk_norm_rope_write(self, qkv, positions, slots, q_weight, k_weight, inv_freq, rotary_dim, eps, kv_layer,
+    def rope_table(self, positions, inv_freq):
+        ang = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).double()  # float32 product
+        return torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).to(torch.float32)
+
+    def qk_norm_rope_write(self, qkv, slots, q_weight, k_weight, cos_sin, rotary_dim, eps, kv_layer,
                            num_q_heads, num_kv_heads, head_dim, write_kv=True):
         nq, nkv, d = num_q_heads, num_kv_heads, head_dim
         N = qkv.shape[0]
@@ -65,8 +69,7 @@ class TorchOps:
             if rotary_dim == 0:
                 return t
             half = rotary_dim // 2
-            ang = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).to(self.cd)  # float32 product
-            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            c, s = cos_sin[:, None, :, 0].to(self.cd), cos_sin[:, None, :, 1].to(self.cd)
             x1, x2 = t[..., :half], t[..., half:rotary_dim]
             return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, t[..., rotary_dim:]], dim=-1)
 
