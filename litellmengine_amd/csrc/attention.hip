@@ -17,7 +17,7 @@
 // Kernels:
 //  * paged_attention_generic_kernel: any type, head size <= 256, page size,
 //    window; one workgroup per (token, q head).  The 32-bit path and odd sizes.
-//  * mfma_decode_kernel / mfma_combine_kernel: bfloat16, head size a multiple of
+//  * mfma_decode_kernel (+ mfma_combine_kernel): bfloat16, head size a multiple of
 //    32, page size a multiple of 16.  One workgroup per (request, kv head, key
 //    split); the q heads of the group (and up to 16 / group tokens) are the 16
 //    columns of v_mfma_f32_16x16x32_bf16 tiles, so every K/V byte is read once
@@ -336,8 +336,8 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
-    float* __restrict__ ws_ml, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
-    float scale_log2) {
+    float* __restrict__ ws_ml, int ws_stride, int nq, int nkv, int P, int64_t page_stride, int max_pages,
+    int window, float scale_log2) {
     constexpr int D = DK * 32;
     extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
     float* s_o = smem;
@@ -395,42 +395,45 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
         if (nsplit == 1) {
             out[head_row * D + e] = (bf16_t)(num / den);
         } else {
-            ws_o[(head_row * nsplit + split) * D + e] = num;
+            ws_o[(head_row * ws_stride + split) * D + e] = num;
             if (e == 0) {
-                ws_ml[(head_row * nsplit + split) * 2] = big;
-                ws_ml[(head_row * nsplit + split) * 2 + 1] = den;
+                ws_ml[(head_row * ws_stride + split) * 2] = big;
+                ws_ml[(head_row * ws_stride + split) * 2 + 1] = den;
             }
         }
     }
 }
 
-// merges the splits of mfma_decode_kernel.  grid = (tokens, q heads), one wavefront each;
-// lane k holds (m, l) of split k (nsplit <= 64).  `mixed` != 0: the batch also holds
-// requests of the prefill kernel, whose tokens are left alone.
+// Merges the key splits.  grid = (tokens, q heads), one wavefront each; lane k holds (m, l) of
+// split k (at most 64 splits).  A token of a request with at most 16 rows was split
+// `nsplit_decode` ways by the decode kernel, any other `nsplit_prefill` ways by the prefill
+// kernel; a token whose kernel did not split was written by that kernel itself.
 __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __restrict__ ws_o,
-                                                                const float* __restrict__ ws_ml,
+                                                                const float* __restrict__ ws_ml, int ws_stride,
                                                                 const int32_t* __restrict__ cu_tokens,
                                                                 const int32_t* __restrict__ token_seq,
                                                                 bf16_t* __restrict__ out, int nq, int nkv, int D,
-                                                                int nsplit, int mixed) {
+                                                                int nsplit_decode, int nsplit_prefill) {
     const int64_t tok = blockIdx.x;
     const int h = blockIdx.y;
-    if (mixed) {
+    int nsplit = nsplit_decode;
+    if (nsplit_decode != nsplit_prefill) {
         const int s = token_seq[tok];
-        if ((cu_tokens[s + 1] - cu_tokens[s]) * (nq / nkv) > 16) return;
+        if ((cu_tokens[s + 1] - cu_tokens[s]) * (nq / nkv) > 16) nsplit = nsplit_prefill;
     }
+    if (nsplit <= 1) return;
     const int lane = threadIdx.x;
     const int64_t head_row = tok * nq + h;
     float m = NEG_BIG, l = 0.f;
     if (lane < nsplit) {
-        const float2 ml = *(const float2*)(ws_ml + (head_row * nsplit + lane) * 2);
+        const float2 ml = *(const float2*)(ws_ml + (head_row * ws_stride + lane) * 2);
         m = ml.x;
         l = ml.y;
     }
     const float big = wave_max(m);
     const float f = exp2f(m - big);  // 0 for lanes without a split (l = 0 there anyway)
     const float den = wave_sum(l * f);
-    const float* o = ws_o + head_row * nsplit * D;
+    const float* o = ws_o + head_row * ws_stride * D;
     for (int e = lane; e < D; e += LLE_WAVE) {
         float num = 0.f;
         for (int k = 0; k < nsplit; ++k) num += o[(int64_t)k * D + e] * __shfl(f, k, LLE_WAVE);
@@ -438,8 +441,9 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     }
 }
 
-// Requests with more than 16 rows.  grid = (row blocks of 128, kv heads, requests); each
-// wavefront owns 32 rows.  The 32-key tiles of K and V^T are copied from the pages into LDS
+// Requests with more than 16 rows.  grid = (row blocks of 128 x key splits, kv heads, requests);
+// each wavefront owns 32 rows.  A short portion after a long past has few row blocks: its keys
+// are then split over `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K and V^T are copied from the pages into LDS
 // once per workgroup (all 256 threads, the next tile while this one is multiplied) and every
 // wavefront reads its matrix-core operands from there: 128 rows share one pass over the keys.
 //   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
@@ -450,8 +454,9 @@ template <int DK>
 __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
-    const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, int nq, int nkv, int P, int64_t page_stride,
-    int max_pages, int window, float scale_log2) {
+    const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, int ws_stride, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages,
+    int window, float scale_log2) {
     constexpr int D = DK * 32;
     constexpr int PRE_RT = PRE_RT_OF(DK);
     constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT;
@@ -467,7 +472,9 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
     const int nrows = q_len * G;
     if (nrows <= 16) return;  // the decode kernel's
     // the last rows see the most keys: they are started first
-    const int block_row0 = (gridDim.x - 1 - blockIdx.x) * PRE_ROWS;
+    const int row_blocks = gridDim.x / nsplit;
+    const int split = blockIdx.x / row_blocks;
+    const int block_row0 = (row_blocks - 1 - blockIdx.x % row_blocks) * PRE_ROWS;
     if (block_row0 >= nrows) return;
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
@@ -480,7 +487,12 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
     const int hi = past + block_last_row / G;
     const int block_first_pos = past + block_row0 / G;
     const int lo_min = window > 0 ? max(0, block_first_pos - window + 1) : 0;
-    const int first_step = lo_min / KSTEP, end_step = hi / KSTEP + 1;
+    int first_step = lo_min / KSTEP, end_step = hi / KSTEP + 1;
+    if (nsplit > 1) {  // this workgroup's share of the steps (it may be empty)
+        const int per_split = (end_step - first_step + nsplit - 1) / nsplit;
+        first_step = first_step + split * per_split;
+        end_step = min(end_step, first_step + per_split);
+    }
 
     const int row0 = block_row0 + wave * (16 * PRE_RT);
     RowInfo row[PRE_RT];
@@ -545,8 +557,10 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
         }
     };
 
-    fetch(first_step);
-    stash(0);
+    if (first_step < end_step) {
+        fetch(first_step);
+        stash(0);
+    }
     __syncthreads();
     for (int step = first_step; step < end_step; ++step) {
         const int buf = (step - first_step) & 1;
@@ -572,7 +586,18 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
         const int r = row0 + 16 * t + r16;
         if (r >= nrows) continue;
         const int tk = r / G, g = r - tk * G;
-        bf16_t* dst = out + ((int64_t)(q_start + tk) * nq + kvh * G + g) * D;
+        const int64_t head_row = (int64_t)(q_start + tk) * nq + kvh * G + g;
+        if (nsplit > 1) {
+            float* po = ws_o + (head_row * ws_stride + split) * D;
+#pragma unroll
+            for (int n = 0; n < 2 * DK; ++n) *(f32x4*)(po + 16 * n + 4 * c) = st.o[t][n];
+            if (c == 0) {
+                ws_ml[(head_row * ws_stride + split) * 2] = st.m[t];
+                ws_ml[(head_row * ws_stride + split) * 2 + 1] = st.l[t];
+            }
+            continue;
+        }
+        bf16_t* dst = out + head_row * D;
         const float inv = 1.0f / st.l[t];
 #pragma unroll
         for (int n = 0; n < 2 * DK; ++n) {
@@ -589,9 +614,13 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
                        const int32_t* seq_slots, const int32_t* cu_tokens, const int32_t* kv_lens,
                        const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
                        int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
-                       int run_decode, int nsplit, int run_prefill, int max_q_len, hipStream_t stream) {
+                       int run_decode, int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
+                       hipStream_t stream) {
     constexpr int D = DK * 32;
     const int G = nq / nkv;
+    if (!run_decode) nsplit_decode = 1;
+    if (!run_prefill) nsplit_prefill = 1;
+    const int ws_stride = nsplit_decode > nsplit_prefill ? nsplit_decode : nsplit_prefill;
     if (run_decode) {
         const size_t smem = (size_t)(DEC_WAVES * 16 * D + 2 * DEC_WAVES * 16) * sizeof(float);
         if (smem > 64 * 1024) {
@@ -599,45 +628,49 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e != hipSuccess) return (int)e;
         }
-        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit), DEC_WAVES * LLE_WAVE, smem, stream>>>(
-            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, nq, nkv, P, page_stride,
-            max_pages, window, scale_log2);
-        if (nsplit > 1)
-            mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(ws_o, ws_ml, cu_tokens, token_seq, out, nq, nkv,
-                                                                      D, nsplit, run_prefill);
+        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit_decode), DEC_WAVES * LLE_WAVE, smem, stream>>>(
+            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nq, nkv, P,
+            page_stride, max_pages, window, scale_log2);
     }
     if (run_prefill) {
-        const int rows = max_q_len * G;
         constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT_OF(DK);
+        const int rows = max_q_len * G;
         const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
-        mfma_prefill_kernel<DK><<<dim3(blocks, nkv, S), ATT_WAVES * LLE_WAVE, 0, stream>>>(
-            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, nq, nkv, P, page_stride, max_pages, window,
-            scale_log2);
+        mfma_prefill_kernel<DK><<<dim3(blocks * nsplit_prefill, nkv, S), ATT_WAVES * LLE_WAVE, 0, stream>>>(
+            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill, nq,
+            nkv, P, page_stride, max_pages, window, scale_log2);
     }
+    if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
+        mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(
+            ws_o, ws_ml, ws_stride, cu_tokens, token_seq, out, nq, nkv, D, run_decode ? nsplit_decode : nsplit_prefill,
+            run_prefill ? nsplit_prefill : nsplit_decode);
     return (int)hipGetLastError();
 }
 
 // bfloat16, head_dim a multiple of 32 (<= 256), page size a multiple of 16.
 // run_decode / run_prefill say which kinds of request the batch holds (requests
-// with q_len * group <= 16 rows are the decode kernel's); nsplit > 1 needs the
-// workspaces ws_o [N * nq * nsplit * d] and ws_ml [N * nq * nsplit * 2] floats.
+// with q_len * group <= 16 rows are the decode kernel's); with ns = max(nsplit_decode,
+// nsplit_prefill) > 1 the workspaces ws_o [N * nq * ns * d] and ws_ml [N * nq * ns * 2]
+// floats are needed (ns <= 64).
 extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, const void* block_tables,
                                         const void* seq_slots, const void* cu_tokens, const void* kv_lens,
                                         const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
                                         int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
-                                        int window, float scale, int run_decode, int nsplit, int run_prefill,
-                                        int max_q_len, hipStream_t stream) {
+                                        int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
+                                        int nsplit_prefill, int max_q_len, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv > 65535) return (int)hipErrorInvalidValue;
+    if (nsplit_decode < 1 || nsplit_decode > 64 || nsplit_prefill < 1 || nsplit_prefill > 64)
+        return (int)hipErrorInvalidValue;
     const float scale_log2 = scale * 1.44269504088896340736f;
 #define LLE_ATT_CASE(DKV)                                                                                          \
     case DKV:                                                                                                      \
         return launch_mfma<DKV>((const bf16_t*)q, (const bf16_t*)kv_layer, (const int32_t*)block_tables,            \
                                 (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
                                 (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
-                                page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit,          \
-                                run_prefill, max_q_len, stream);
+                                page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit_decode,   \
+                                run_prefill, nsplit_prefill, max_q_len, stream);
     switch (d / 32) {
         LLE_ATT_CASE(1)
         LLE_ATT_CASE(2)

@@ -239,18 +239,19 @@ class HipOps:
         min_q_len = min_q_len or 1
         run_decode = min_q_len * group <= 16
         run_prefill = max_q_len * group > 16
-        nsplit, ws_o, ws_ml = 1, None, None
-        if run_decode:
-            nsplit = self.decode_splits(S, nkv, max_kv_len, win)
-            if nsplit > 1:
-                ws_o = torch.empty((N * nq * nsplit * d,), dtype=torch.float32, device=q.device)
-                ws_ml = torch.empty((N * nq * nsplit * 2,), dtype=torch.float32, device=q.device)
+        ns_decode = self.decode_splits(S, nkv, max_kv_len, win) if run_decode else 1
+        ns_prefill = self.prefill_splits(S, nkv, group, d, max_q_len, max_kv_len, win) if run_prefill else 1
+        ns = max(ns_decode, ns_prefill)
+        ws_o = ws_ml = None
+        if ns > 1:
+            ws_o = torch.empty((N * nq * ns * d,), dtype=torch.float32, device=q.device)
+            ws_ml = torch.empty((N * nq * ns * 2,), dtype=torch.float32, device=q.device)
         self._run("attention", "lle_paged_attention_mfma",
-                  [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _I, _I, _P],
+                  [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _I, _I, _I, _P],
                   _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
                   _ptr(token_seq), _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size,
-                  kv_layer.stride(0), block_table.shape[1], win, float(scale), int(run_decode), nsplit,
-                  int(run_prefill), max_q_len)
+                  kv_layer.stride(0), block_table.shape[1], win, float(scale), int(run_decode), ns_decode,
+                  int(run_prefill), ns_prefill, max_q_len)
         return out
 
     force_generic_attention = False  # tests flip this to compare the two families of kernels
@@ -258,6 +259,20 @@ class HipOps:
     # wavefront) per split are best; more splits cost more in partial results than they gain
     DECODE_TARGET_BLOCKS = 256
     DECODE_MIN_STEPS_PER_SPLIT = 16
+
+    PREFILL_MIN_STEPS_PER_SPLIT = 8
+
+    def prefill_splits(self, num_seqs: int, num_kv_heads: int, group: int, head_dim: int, max_q_len: int,
+                       max_kv_len: int, window: int) -> int:
+        """Key splits of the prompt-portion kernel: 1 unless the portions are so short that
+        their row blocks alone leave most of the chip idle (a tail of a prompt after a long past)."""
+        rows_per_block = 128 if head_dim <= 128 else 64
+        blocks = ((max_q_len * group + rows_per_block - 1) // rows_per_block) * num_kv_heads * max(1, num_seqs)
+        span = min(max_kv_len, window + max_q_len) if window else max_kv_len
+        steps = (span + 31) // 32
+        by_work = max(1, steps // self.PREFILL_MIN_STEPS_PER_SPLIT)
+        by_fill = max(1, self.DECODE_TARGET_BLOCKS // blocks)
+        return int(min(by_work, by_fill, 64))
 
     def decode_splits(self, num_seqs: int, num_kv_heads: int, max_kv_len: int, window: int) -> int:
         """Key splits of the decode kernel: enough workgroups to fill the chip, but

@@ -257,6 +257,8 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
     [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
     [(0, 150), (100, 70)],                        # prompt portions only, one after a past
     [(1200, 3), (64, 64), (15, 1)],
+    [(2000, 49)],                                 # a short tail after a long past: keys split over workgroups
+    [(1500, 40), (1900, 1), (3, 30)],
 ])
 def test_matrix_core_attention(nq, nkv, d, P, window, lens):
     """The bfloat16 matrix-core kernels against the plain form and the generic kernel."""
