@@ -134,3 +134,36 @@ def test_qwen3_8b_layer_sizes(tmp_path):
             assert err < tol, (dtype, cuts, err)
         del runner
         torch.cuda.empty_cache()
+
+
+def test_graph_replays_with_library_products(tmp_path):
+    """Decode steps of 24 requests at the Qwen3-8B layer widths: more rows than the
+    weight-streaming kernel takes, so the captured graph holds library matrix products.
+    Every replay is compared with the same step run without a graph."""
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.models import random_model
+
+    cfg = Qwen3Config.from_dict(dict(
+        architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_size=4096, num_attention_heads=32,
+        num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=32000, rope_theta=1e6,
+        rms_norm_eps=1e-6, tie_word_embeddings=True))
+    model = random_model(cfg, seed=5, dtype="bfloat16")
+    B = 24
+    prompts = [random_tokens(30 + 3 * i, cfg.vocab_size, 200 + i) for i in range(B)]
+    feed = [random_tokens(8, cfg.vocab_size, 300 + i) for i in range(B)]
+    outs = {}
+    for use_graphs in (True, False):
+        cache = CacheManager(model, page_size=16, num_pages=B * 8, max_requests=B, dtype=model.ctx.dtype,
+                             device=model.ctx.device)
+        runner = ModelRunner(model, cache, use_graphs=use_graphs)
+        slots = [runner.admit() for _ in range(B)]
+        runner.step([StepEntry(s, p) for s, p in zip(slots, prompts)])
+        got = []
+        for t in range(8):
+            got.append(runner.step([StepEntry(s, [feed[i][t]], [0]) for i, s in enumerate(slots)]).float().cpu())
+            if t == 3:  # eager work between replays
+                extra = runner.admit() if cache.num_free_slots else None
+        outs[use_graphs] = torch.stack(got)
+    diff = (outs[True] - outs[False]).abs().max().item()
+    assert diff < 2e-2, diff
+    assert torch.isfinite(outs[True]).all()

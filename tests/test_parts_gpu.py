@@ -1,7 +1,8 @@
 """Each model part alone against the plain implementation, and a toy
 architecture defined HERE (a mixer with state of its own, another position
-encoding, a block that runs twice, a layer that reads another layer's cache)
-that is registered, built and stepped without any change to the package."""
+encoding, a feed-forward with routing, a block that runs twice, a layer that
+reads another layer's cache) that is registered, built and stepped without any
+change to the package."""
 import dataclasses
 import math
 
@@ -12,8 +13,8 @@ from litellmengine_amd.cache import CacheManager
 from litellmengine_amd.config import register_architecture
 from litellmengine_amd.engine import ModelRunner, StepEntry
 from litellmengine_amd.models import DecoderLM, PlanEntry, make_context, random_model
-from litellmengine_amd.parts import (Embedding, GatedMLP, Linear, Mixer, PagedAttention, PositionEncoding,
-                                     PreNormBlock, RMSNorm, RotaryHalfSplit, StateSpec)
+from litellmengine_amd.parts import (Embedding, FeedForward, GatedMLP, Linear, Mixer, PagedAttention,
+                                     PositionEncoding, PreNormBlock, RMSNorm, RotaryHalfSplit, StateSpec)
 from litellmengine_amd.weights import TensorSpec, random_weights
 from tests.plain import qwen3_plain as plain
 from tests.tiny import random_tokens
@@ -151,6 +152,42 @@ class LearnedAdditivePosition(PositionEncoding):
         return q + t, k + t
 
 
+class TopOneRoutedFF(FeedForward):
+    """A feed-forward with routing: router logits in 32-bit, every token goes to its best
+    expert (a plain two-layer perceptron with SiLU), scaled by that expert's probability."""
+
+    def __init__(self, prefix, hidden, width, experts):
+        self.prefix, self.hidden, self.width, self.experts = prefix, hidden, width, experts
+
+    def tensor_specs(self):
+        specs = {self.prefix + "router": TensorSpec((self.experts, self.hidden))}
+        for e in range(self.experts):
+            specs[f"{self.prefix}e{e}.up"] = TensorSpec((self.width, self.hidden))
+            specs[f"{self.prefix}e{e}.down"] = TensorSpec((self.hidden, self.width))
+        return specs
+
+    def bind(self, weights, ctx):
+        self.ctx = ctx
+        self.router = weights[self.prefix + "router"].float() * ROUTER_GAIN
+        self.up = [weights[f"{self.prefix}e{e}.up"].to(ctx.dtype).contiguous() for e in range(self.experts)]
+        self.down = [weights[f"{self.prefix}e{e}.down"].to(ctx.dtype).contiguous() for e in range(self.experts)]
+
+    def forward(self, x):
+        probs = torch.softmax(x.float() @ self.router.t(), dim=-1)
+        best = probs.argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for e in range(self.experts):
+            rows = (best == e).nonzero().flatten()
+            if rows.numel():
+                h = torch.nn.functional.silu(self.ctx.ops.linear(x[rows].contiguous(), self.up[e]).float()).to(x.dtype)
+                y = self.ctx.ops.linear(h, self.down[e]).float() * probs[rows, e][:, None]
+                out[rows] = y.to(x.dtype)
+        return out
+
+
+ROUTER_GAIN = 40.0  # wide margins between the experts' logits, so that rounding does not re-route a token
+
+
 class AttentionWithPosition(PagedAttention):
     def tensor_specs(self):
         return {**super().tensor_specs(), **self.position.tensor_specs()}
@@ -181,8 +218,8 @@ def build_toy(c: ToyConfig) -> DecoderLM:
                                      qk_norm_eps=c.eps)
 
     def block(i, mixer):
-        return PreNormBlock(RMSNorm(f"l{i}.n1", c.hidden_size, c.eps), mixer, RMSNorm(f"l{i}.n2", c.hidden_size, c.eps),
-                            GatedMLP(f"l{i}.mlp.", c.hidden_size, c.ffn))
+        ff = TopOneRoutedFF(f"l{i}.moe.", c.hidden_size, c.ffn, 3) if i == 2 else GatedMLP(f"l{i}.mlp.", c.hidden_size, c.ffn)
+        return PreNormBlock(RMSNorm(f"l{i}.n1", c.hidden_size, c.eps), mixer, RMSNorm(f"l{i}.n2", c.hidden_size, c.eps), ff)
 
     blocks = [block(0, RunningMeanMixer("l0.mean.weight", c.hidden_size)), block(1, attention(1)), block(2, attention(2))]
     # block 0 runs twice (its second run has state of its own); block 2 reads the keys and values of block 1
@@ -196,6 +233,14 @@ def toy_plain(ids, w, c: ToyConfig):
     n = lambda x, name: plain.rms_norm(x, w[name], c.eps)
 
     def mlp(x, i):
+        if i == 2:  # routed: best expert by router logits, scaled by its probability
+            probs = torch.softmax(plain.linear(x, w["l2.moe.router"] * ROUTER_GAIN), dim=-1)
+            out = torch.zeros_like(x)
+            for t in range(x.shape[0]):
+                e = int(probs[t].argmax())
+                h = torch.nn.functional.silu(plain.linear(x[t : t + 1], w[f"l2.moe.e{e}.up"]))
+                out[t] = plain.linear(h, w[f"l2.moe.e{e}.down"])[0] * probs[t, e]
+            return out
         return plain.gated_mlp(x, w[f"l{i}.mlp.gate_proj.weight"], w[f"l{i}.mlp.up_proj.weight"], w[f"l{i}.mlp.down_proj.weight"])
 
     def mean_block(x):
