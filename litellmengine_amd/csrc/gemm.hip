@@ -1,9 +1,9 @@
 // Matrix products C[M, N] = A[M, K] . B[N, K]^T (weights are [out, in] row-major
 // like the reference's Linear, src/layers/linear.cu:169-215, which calls
 // cublasSgemm).  This file holds the true 32-bit product (plain FMA, no matrix
-// cores, no reduced-precision mode) and 16-bit-in / 32-bit-accumulate variants
-// of the same tiling; the sum over k runs in index order whatever M is, so a
-// row's result does not depend on what else is in the batch.
+// cores, no reduced-precision mode; the sum over k runs in index order whatever
+// M is, so a row's result does not depend on what else is in the batch) and the
+// bfloat16 weight-streaming product of decoding.
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -62,23 +62,15 @@ __global__ __launch_bounds__(256) void gemm_nt_simt_kernel(const TA* __restrict_
     }
 }
 
-// in_dtype: type of A and B; out_dtype: type of C
+// float32 in, float32 out (in_dtype and out_dtype must say so)
 extern "C" int lle_gemm_nt_simt(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda,
                                 int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (in_dtype != LLE_F32 || out_dtype != LLE_F32) return (int)hipErrorInvalidValue;
     dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM);
     if (grid.y > 65535) return (int)hipErrorInvalidValue;
-    if (in_dtype == LLE_F32 && out_dtype == LLE_F32)
-        gemm_nt_simt_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)A, (const float*)B, (float*)C, M,
-                                                                     N, K, lda, ldb, ldc);
-    else if (in_dtype == LLE_BF16 && out_dtype == LLE_F32)
-        gemm_nt_simt_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)B, (float*)C,
-                                                                      M, N, K, lda, ldb, ldc);
-    else if (in_dtype == LLE_BF16 && out_dtype == LLE_BF16)
-        gemm_nt_simt_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)B,
-                                                                       (bf16_t*)C, M, N, K, lda, ldb, ldc);
-    else
-        return (int)hipErrorInvalidValue;
+    gemm_nt_simt_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)A, (const float*)B, (float*)C, M, N, K,
+                                                                 lda, ldb, ldc);
     LLE_RETURN_LAUNCH_STATUS();
 }
 

@@ -125,25 +125,25 @@ class HipOps:
     def linear(self, x, weight, out_dtype=None) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
         kernel (a true 32-bit product).  bfloat16 operands: few rows take the
-        weight-streaming matrix-core kernel (either result type, up to 64 rows for a
-        float32 result); more rows go to the library product (bfloat16 result) or the
-        32-bit-accumulate kernel (float32 result)."""
+        weight-streaming matrix-core kernel, more rows the library product; both
+        accumulate in 32-bit and write either result type."""
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape
         N = weight.shape[0]
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
         out_dtype = out_dtype or x.dtype
-        skinny = x.dtype == torch.bfloat16 and K % 8 == 0 and not self.force_library_gemm and (
-            M <= self.SKINNY_MAX_ROWS or (out_dtype == torch.float32 and M <= 64)
-            or (M <= 16 and N * K <= self.SKINNY_SMALL_WEIGHT))
-        if skinny:
-            out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-            self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
-                      _ptr(x), _ptr(weight), _ptr(out), M, N, K, dtype_code(out_dtype))
-            return out
-        if x.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
-            return torch.mm(x, weight.t())
+        if x.dtype == torch.bfloat16:
+            skinny = K % 8 == 0 and not self.force_library_gemm and (
+                M <= self.SKINNY_MAX_ROWS or (M <= 16 and N * K <= self.SKINNY_SMALL_WEIGHT))
+            if skinny:
+                out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+                self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
+                          _ptr(x), _ptr(weight), _ptr(out), M, N, K, dtype_code(out_dtype))
+                return out
+            # the library product accumulates in 32-bit and can leave the result so
+            return torch.mm(x, weight.t()) if out_dtype == torch.bfloat16 else torch.mm(x, weight.t(), out_dtype=out_dtype)
+        _need(out_dtype == torch.float32, "a float32 product has a float32 result")
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
         self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
