@@ -27,6 +27,7 @@
 //    all keys up to each row's own position; the four wavefronts of a workgroup
 //    share the K/V tiles through LDS.
 #include "common.h"
+#include <type_traits>
 
 LLE_DEFINE_ERROR_STRING()
 
@@ -449,9 +450,15 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 //   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
 //   LDS V^T tile: [D][32 keys + 4]
 // row tiles per wavefront: two while the accumulators fit the register file
-#define PRE_RT_OF(DK) ((DK) <= 4 ? 2 : 1)
+#ifndef PRE_WAVES
+#define PRE_WAVES 8
+#endif
+#ifndef PRE_RT_MAX
+#define PRE_RT_MAX 2
+#endif
+#define PRE_RT_OF(DK) ((DK) <= 4 ? PRE_RT_MAX : 1)
 template <int DK>
-__global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_prefill_kernel(
+__global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
@@ -459,7 +466,7 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
     int window, float scale_log2) {
     constexpr int D = DK * 32;
     constexpr int PRE_RT = PRE_RT_OF(DK);
-    constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT;
+    constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
     constexpr int KROW = D + 8;       // elements per key row in LDS
     constexpr int VROW = KSTEP + 4;   // elements per value-element row in LDS
     constexpr int TILE = KSTEP * KROW + D * VROW;
@@ -512,9 +519,12 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
     const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
     // a tile holds 4 D 16-byte pieces of K and as many of V^T; this thread copies NP of each
     constexpr int PIECES = 4 * D;
-    constexpr int NP = (PIECES + ATT_WAVES * LLE_WAVE - 1) / (ATT_WAVES * LLE_WAVE);
-    bf16x8 stage_k[NP], stage_v[NP];
-    auto fetch = [&](int step) {
+    constexpr int NP = (PIECES + PRE_WAVES * LLE_WAVE - 1) / (PRE_WAVES * LLE_WAVE);
+    // two tiles are on their way from memory at any time (register sets 0 and 1); a tile is
+    // written to LDS one step after its loads were issued and multiplied one step later still
+    bf16x8 stage_k[2][NP], stage_v[2][NP];
+    auto fetch = [&](int step, auto set_c) {
+        constexpr int set = decltype(set_c)::value;
         const int j0 = step * KSTEP;
         const bf16_t* page[2];
         int off[2];
@@ -527,45 +537,42 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
         }
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
-            const int piece = threadIdx.x + ATT_WAVES * LLE_WAVE * i;
+            const int piece = threadIdx.x + PRE_WAVES * LLE_WAVE * i;
             if (piece < PIECES) {
                 const int key = piece / (D / 8), ch = piece % (D / 8);  // key 0..31, 16-byte piece of its row
                 const int xk = key / 16;
-                stage_k[i] = *(const bf16x8*)((xk ? page[1] : page[0]) + k_head +
-                                              (int64_t)((xk ? off[1] : off[0]) + key % 16) * D + ch * 8);
+                stage_k[set][i] = *(const bf16x8*)((xk ? page[1] : page[0]) + k_head +
+                                                   (int64_t)((xk ? off[1] : off[0]) + key % 16) * D + ch * 8);
                 const int dd = piece / 4, part = piece % 4;  // value element 0..D-1, quarter of its 32 keys
                 const int xv = part / 2;
-                stage_v[i] = *(const bf16x8*)((xv ? page[1] : page[0]) + v_head + (int64_t)dd * P +
-                                              (xv ? off[1] : off[0]) + (part % 2) * 8);
+                stage_v[set][i] = *(const bf16x8*)((xv ? page[1] : page[0]) + v_head + (int64_t)dd * P +
+                                                   (xv ? off[1] : off[0]) + (part % 2) * 8);
             }
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, auto set_c) {
+        constexpr int set = decltype(set_c)::value;
         bf16_t* kt = lds + buf * TILE;
         bf16_t* vt = kt + KSTEP * KROW;
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
-            const int piece = threadIdx.x + ATT_WAVES * LLE_WAVE * i;
+            const int piece = threadIdx.x + PRE_WAVES * LLE_WAVE * i;
             if (piece < PIECES) {
                 const int key = piece / (D / 8), ch = piece % (D / 8);
-                *(bf16x8*)(kt + key * KROW + ch * 8) = stage_k[i];
+                *(bf16x8*)(kt + key * KROW + ch * 8) = stage_k[set][i];
                 const int dd = piece / 4, part = piece % 4;
                 bf16_t* dst = vt + dd * VROW + (part / 2) * 16 + (part % 2) * 8;  // 8-byte aligned
-                *(bf16x4*)dst = __builtin_shufflevector(stage_v[i], stage_v[i], 0, 1, 2, 3);
-                *(bf16x4*)(dst + 4) = __builtin_shufflevector(stage_v[i], stage_v[i], 4, 5, 6, 7);
+                *(bf16x4*)dst = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 0, 1, 2, 3);
+                *(bf16x4*)(dst + 4) = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 4, 5, 6, 7);
             }
         }
     };
-
-    if (first_step < end_step) {
-        fetch(first_step);
-        stash(0);
-    }
-    __syncthreads();
-    for (int step = first_step; step < end_step; ++step) {
-        const int buf = (step - first_step) & 1;
-        const bool more = step + 1 < end_step;
-        if (more) fetch(step + 1);
+    // one step: tile `step` is in LDS buffer `buf`; tile step + 1 sits in register set `set`
+    // (loads issued a step ago) and goes to the other buffer; tile step + 2 is requested now
+    // into the other register set
+    auto one_step = [&](int step, int buf, auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+        if (step + 2 < end_step) fetch(step + 2, std::integral_constant<int, 1 - set>{});
         if (step >= my_first && step < my_end) {
             const bf16_t* kt = lds + buf * TILE;
             const bf16_t* vt = kt + KSTEP * KROW;
@@ -577,8 +584,19 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE, DK <= 4 ? 2 : 1) void mfma_pre
                 },
                 step * KSTEP, scale_log2);
         }
-        if (more) stash(buf ^ 1);
+        if (step + 1 < end_step) stash(buf ^ 1, set_c);
         __syncthreads();
+    };
+
+    if (first_step < end_step) {
+        fetch(first_step, std::integral_constant<int, 0>{});
+        if (first_step + 1 < end_step) fetch(first_step + 1, std::integral_constant<int, 1>{});
+        stash(0, std::integral_constant<int, 0>{});
+    }
+    __syncthreads();
+    for (int step = first_step; step < end_step; step += 2) {
+        one_step(step, 0, std::integral_constant<int, 1>{});
+        if (step + 1 < end_step) one_step(step + 1, 1, std::integral_constant<int, 0>{});
     }
     finish_rows<DK, PRE_RT>(st);
 #pragma unroll
@@ -633,10 +651,10 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
             page_stride, max_pages, window, scale_log2);
     }
     if (run_prefill) {
-        constexpr int PRE_ROWS = ATT_WAVES * 16 * PRE_RT_OF(DK);
+        constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT_OF(DK);
         const int rows = max_q_len * G;
         const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
-        mfma_prefill_kernel<DK><<<dim3(blocks * nsplit_prefill, nkv, S), ATT_WAVES * LLE_WAVE, 0, stream>>>(
+        mfma_prefill_kernel<DK><<<dim3(blocks * nsplit_prefill, nkv, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
             q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill, nq,
             nkv, P, page_stride, max_pages, window, scale_log2);
     }
