@@ -167,3 +167,42 @@ def test_graph_replays_with_library_products(tmp_path):
     diff = (outs[True] - outs[False]).abs().max().item()
     assert diff < 2e-2, diff
     assert torch.isfinite(outs[True]).all()
+
+
+ODD = [
+    # head size 80 (no matrix-core attention), width not a multiple of 4, odd vocabulary, page size 3
+    dict(num_hidden_layers=2, hidden_size=102, num_attention_heads=5, num_key_value_heads=5, head_dim=80,
+         intermediate_size=150, vocab_size=1001, rope_theta=3e4, rms_norm_eps=2e-6, tie_word_embeddings=True, page=3),
+    # one kv head for seven q heads, head size 64, page size 32, widths that are multiples of 2 only
+    dict(num_hidden_layers=1, hidden_size=70, num_attention_heads=7, num_key_value_heads=1, head_dim=64,
+         intermediate_size=94, vocab_size=333, rope_theta=1e6, rms_norm_eps=1e-5, tie_word_embeddings=False, page=32),
+    # head size 256, a window of 9 on every layer, page size 1
+    dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=2, num_key_value_heads=2, head_dim=256,
+         intermediate_size=72, vocab_size=50, rope_theta=1e4, rms_norm_eps=1e-6, tie_word_embeddings=False,
+         sliding_window=9, layer_types=["sliding_attention", "sliding_attention"], page=1),
+    # head size 96 (matrix cores, three 32-element steps), group of 3, page size 48
+    dict(num_hidden_layers=2, hidden_size=96, num_attention_heads=6, num_key_value_heads=2, head_dim=96,
+         intermediate_size=136, vocab_size=257, rope_theta=5e5, rms_norm_eps=1e-6, tie_word_embeddings=True, page=48),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("index", range(len(ODD)))
+def test_odd_sizes(tmp_path, index, dtype):
+    """Sizes that push the kernels off their fast paths (or onto rarely used ones)."""
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.weights import write_model_dir
+
+    spec = dict(ODD[index])
+    page = spec.pop("page")
+    cfg = Qwen3Config.from_dict(dict(spec, architectures=["Qwen3ForCausalLM"]))
+    d = str(tmp_path / f"odd{index}")
+    write_model_dir(cfg, d, 21 + index, torch.bfloat16)
+    pcfg, w = plain.read_model_dir(d)
+    tokens = random_tokens(50, cfg.vocab_size, 9)
+    want = plain.model_logits_fast(tokens, w, pcfg)
+    runner = make_runner(d, dtype, page, 64 // page + 2)
+    for cuts in ([50], [18] + [1] * 32, [2, 9, 20, 2, 17]):
+        got = run_cut(runner, tokens, cuts)
+        err = (got.double() - want).abs().max().item() / max(1.0, want.abs().max().item())
+        assert err < TOL[dtype], (cuts, err)
