@@ -95,12 +95,43 @@ typedef float gf32x4 __attribute__((ext_vector_type(4)));
 
 // GATED: W holds gate rows [0, N/2) and then up rows [N/2, N); a workgroup takes 16 gate rows
 // and the 16 up rows that go with them (NT = 2) and writes silu(gate) * up, C is [M, N/2].
-template <int MT, int NT, bool GATED, typename TC, int SK_WAVES, int UNROLL>
+//
+// The RMSNorm between two products can be folded into them (up to 16 rows).  With
+//   norm(h)[m][k] = h[m][k] * w[k] * r[m],  r[m] = 1 / sqrt(mean_k h[m][k]^2 + eps)
+// the factor r[m] commutes with the product that follows, so
+//   RESID (the product before the norm): its result is the delta of the residual stream; the
+//     epilogue forms h = hidden + delta in 32-bit, writes it back, writes xw = h * w as the
+//     next product's input, and leaves the sum of h^2 over its 16 columns per row in
+//     ss_part[workgroup][16];
+//   SCALED (the product after the norm): adds up the parts, and multiplies its rows by r[m].
+struct NormFold {
+    float* hidden;          // RESID: residual stream [M, N], read and written
+    const void* weight;     // RESID: norm weight [N]
+    int weight_dtype;
+    bf16_t* xw;             // RESID: out, [M, N]
+    float* ss_out;          // RESID: out, [workgroups][16]
+    const float* ss_in;     // SCALED: [parts][16]
+    int parts;              // SCALED
+    float eps;              // SCALED
+};
+
+template <int MT, int NT, bool GATED, bool RESID, bool SCALED, typename TC, int SK_WAVES, int UNROLL>
 __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                          const bf16_t* __restrict__ W,
-                                                                         TC* __restrict__ C, int M, int N, int K) {
+                                                                         TC* __restrict__ C, int M, int N, int K,
+                                                                         NormFold fold) {
+    static_assert(!(RESID || SCALED) || MT == 1, "the norm is folded for up to 16 rows");
     // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
+    __shared__ float s_inv[16];
+    if (SCALED && threadIdx.x < 256) {  // r[m] from the parts, 16 threads a row
+        const int m = threadIdx.x / 16, j = threadIdx.x % 16;
+        float part = 0.f;
+        for (int b = j; b < fold.parts; b += 16) part += fold.ss_in[b * 16 + m];
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, LLE_WAVE);
+        if (j == 0) s_inv[m] = 1.0f / sqrtf(part / (float)K + fold.eps);
+    }
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
     const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
@@ -194,7 +225,31 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
                 g += s_acc[w][0][mt][n][m];
                 u += s_acc[w][NT - 1][mt][n][m];
             }
+            if (SCALED) {
+                g *= s_inv[m];
+                u *= s_inv[m];
+            }
             C[row * (N / 2) + col] = from_f32<TC>(g / (1.0f + expf(-g)) * u);
+        }
+        return;
+    }
+    if (RESID) {  // NT = MT = 1: thread (m, n) of the first 256 owns element [m][n0 + n]
+        if (threadIdx.x < 256) {
+            const int m = threadIdx.x / 16, n = threadIdx.x % 16;
+            const int64_t col = n0 + n;
+            float sq = 0.f;
+            if (m < M && col < N) {
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][0][n][m];
+                const float h = fold.hidden[(int64_t)m * N + col] + sum;
+                fold.hidden[(int64_t)m * N + col] = h;
+                fold.xw[(int64_t)m * N + col] = (bf16_t)(h * load_as_f32(fold.weight, col, fold.weight_dtype));
+                sq = h * h;
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, LLE_WAVE);
+            if (n == 0) fold.ss_out[(int64_t)blockIdx.x * 16 + m] = sq;
         }
         return;
     }
@@ -205,6 +260,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][nt][mt][n][m];
+        if (SCALED) sum *= s_inv[m];
         C[row * N + col] = from_f32<TC>(sum);
     }
 }
@@ -216,11 +272,12 @@ static int launch_skinny(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, 
     const int per_block = GATED ? 16 : 16 * NT;
     const int blocks = (rows + per_block - 1) / per_block;
     const int mt = (M + 15) / 16;
+    const NormFold none = {};
     switch (mt) {
-        case 1: gemm_skinny_kernel<1, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 2: gemm_skinny_kernel<2, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 3: gemm_skinny_kernel<3, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
-        case 4: gemm_skinny_kernel<4, NT, GATED, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K); break;
+        case 1: gemm_skinny_kernel<1, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
+        case 2: gemm_skinny_kernel<2, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
+        case 3: gemm_skinny_kernel<3, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
+        case 4: gemm_skinny_kernel<4, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();
@@ -247,4 +304,43 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
     if (M <= 0 || N2 <= 0) return 0;
     if (M > 32 || K % 8 != 0 || K <= 0 || N2 % 2 != 0) return (int)hipErrorInvalidValue;
     return launch_skinny<bf16_t, 2, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, stream);
+}
+
+// The product BEFORE a folded norm: delta = X W^T [M, N] is added into `hidden` (float32 [M, N],
+// in place), xw = hidden * norm_weight goes to `xw` (bfloat16 [M, N]) and the sums of squares of
+// the new hidden over each workgroup's 16 columns to ss_part [(N + 15) / 16][16].  1 <= M <= 16.
+extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hidden, const void* norm_weight,
+                                          int weight_dtype, void* xw, void* ss_part, int M, int N, int K,
+                                          hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 != 0 || K <= 0) return (int)hipErrorInvalidValue;
+    NormFold fold = {};
+    fold.hidden = (float*)hidden;
+    fold.weight = norm_weight;
+    fold.weight_dtype = weight_dtype;
+    fold.xw = (bf16_t*)xw;
+    fold.ss_out = (float*)ss_part;
+    gemm_skinny_kernel<1, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
+        (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// The product AFTER a folded norm: X is the xw of lle_gemm_skinny_resid_bf16 and ss_part its
+// `parts` x 16 sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).  gated != 0:
+// W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.  1 <= M <= 16.
+extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C, const void* ss_part, int parts,
+                                           float eps, int M, int N, int K, int gated, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 8 != 0 || K <= 0 || parts <= 0 || (gated && N % 2 != 0)) return (int)hipErrorInvalidValue;
+    NormFold fold = {};
+    fold.ss_in = (const float*)ss_part;
+    fold.parts = parts;
+    fold.eps = eps;
+    if (gated)
+        gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, fold);
+    else
+        gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, fold);
+    LLE_RETURN_LAUNCH_STATUS();
 }

@@ -10,6 +10,7 @@ from typing import Optional
 
 import torch
 
+from ..parts.base import Prenormed
 from . import build
 
 F32, BF16 = 0, 1
@@ -122,11 +123,55 @@ class HipOps:
         return out
 
     # -- matrix products -------------------------------------------------------
-    def linear(self, x, weight, out_dtype=None) -> torch.Tensor:
+    def can_fold_norm(self, rows: int, width: int, dtype) -> bool:
+        """Whether an RMSNorm over `width` of a step of `rows` tokens can be done by the
+        products before and after it (the weight-streaming kernel's few-rows forms)."""
+        return (dtype == torch.bfloat16 and 0 < rows <= self.SKINNY_MAX_ROWS and width % 8 == 0
+                and not self.force_library_gemm)
+
+    def _linear_folded(self, x, weight, fold, gated: bool):
+        """The forms of the weight-streaming product around a folded norm: `x` a Prenormed
+        (its row factors are applied to the result), `fold` a NormFold (the result goes
+        into the residual stream and comes back as the next Prenormed)."""
+        pre = x if isinstance(x, Prenormed) else None
+        xin = pre.xw if pre is not None else x
+        _dev(xin, "x", torch.bfloat16)
+        _dev(weight, "weight", torch.bfloat16)
+        M, K = xin.shape
+        N = weight.shape[0]
+        _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
+        _need(self.can_fold_norm(M, K, xin.dtype), f"a norm cannot be folded into a product of {M} rows of {K}")
+        _need(pre is None or fold is None, "a product takes a Prenormed or makes one, not both")
+        if pre is not None:
+            _dev(pre.sums, "sums", torch.float32)
+            parts = pre.sums.shape[0]
+            _need(pre.sums.shape == (parts, 16) and pre.xw.shape[1] == K, "sums of squares do not fit")
+            _need(not gated or N % 2 == 0, "a gated weight has an even number of rows")
+            out = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=xin.device)
+            self._run("gemm", "lle_gemm_skinny_scaled_bf16", [_P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
+                      _ptr(xin), _ptr(weight), _ptr(out), _ptr(pre.sums), parts, float(pre.eps), M, N, K, int(gated))
+            return out
+        _dev(fold.hidden, "hidden", torch.float32)
+        _dev(fold.weight, "norm weight")
+        _need(not gated and fold.hidden.shape == (M, N) and fold.weight.shape == (N,),
+              f"residual stream {list(fold.hidden.shape)} does not fit a product [{M}, {N}]")
+        _need(self.can_fold_norm(M, N, xin.dtype), f"a norm over {N} cannot be folded")
+        xw = torch.empty((M, N), dtype=torch.bfloat16, device=xin.device)
+        sums = torch.empty(((N + 15) // 16, 16), dtype=torch.float32, device=xin.device)
+        self._run("gemm", "lle_gemm_skinny_resid_bf16", [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+                  _ptr(xin), _ptr(weight), _ptr(fold.hidden), _ptr(fold.weight), dtype_code(fold.weight.dtype),
+                  _ptr(xw), _ptr(sums), M, N, K)
+        return Prenormed(xw, sums, fold.eps)
+
+    def linear(self, x, weight, out_dtype=None, fold=None):
         """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
         kernel (a true 32-bit product).  bfloat16 operands: few rows take the
         weight-streaming matrix-core kernel, more rows the library product; both
-        accumulate in 32-bit and write either result type."""
+        accumulate in 32-bit and write either result type.  `x` a Prenormed or `fold`
+        a NormFold: see _linear_folded."""
+        if fold is not None or isinstance(x, Prenormed):
+            _need(out_dtype in (None, torch.bfloat16), "a product beside a folded norm writes bfloat16")
+            return self._linear_folded(x, weight, fold, gated=False)
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape
@@ -298,6 +343,8 @@ class HipOps:
         """x [M, K], weight [2 I, K] (gate rows, then up rows) -> silu(x gate^T) * (x up^T), [M, I].
         Few bfloat16 rows run as ONE weight-streaming launch with the activation in its
         epilogue; otherwise the product and silu_mul."""
+        if isinstance(x, Prenormed):
+            return self._linear_folded(x, weight, None, gated=True)
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape

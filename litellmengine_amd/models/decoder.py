@@ -106,8 +106,11 @@ class DecoderLM:
         step.scratch.clear()  # per-step tables are made anew in every run (also when a graph is captured)
         hidden = self.embedding.forward(step.token_ids)
         delta = None
+        last = len(self.plan) - 1
         for i, e in enumerate(self.plan):
-            delta = self.blocks[e.block].forward(hidden, delta, step, caches.layer(i))
+            # the norm that the next block starts with, if the products around it may do its work
+            next_norm = self.blocks[self.plan[i + 1].block].entry_norm() if i < last else None
+            delta = self.blocks[e.block].forward(hidden, delta, step, caches.layer(i), next_norm=next_norm)
         if step.logit_rows.shape[0] == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=hidden.device)
         x = self.final_norm.forward(hidden, delta, rows=step.logit_rows)

@@ -1,5 +1,5 @@
 from .attention import PagedAttention
-from .base import Block, BuildContext, FeedForward, KVCacheSpec, Mixer, Norm, Part, PositionEncoding, StateSpec
+from .base import Block, BuildContext, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part, PositionEncoding, Prenormed, StateSpec
 from .block import PreNormBlock
 from .embedding import Embedding
 from .feed_forward import GatedMLP
@@ -9,6 +9,6 @@ from .position import NoPositionEncoding, RotaryHalfSplit
 
 __all__ = [
     "Block", "BuildContext", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
-    "NoPositionEncoding", "Norm", "PagedAttention", "Part", "PositionEncoding", "PreNormBlock", "RMSNorm",
+    "NoPositionEncoding", "Norm", "NormFold", "PagedAttention", "Part", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec",
 ]

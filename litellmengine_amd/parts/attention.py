@@ -25,6 +25,7 @@ from .linear import Linear
 
 class PagedAttention(Mixer):
     graph_safe = True
+    folds_norm = True
 
     def __init__(
         self,
@@ -77,7 +78,7 @@ class PagedAttention(Mixer):
                 qw, kw = qw.float(), kw.float()
             self.q_norm_w, self.k_norm_w = qw.contiguous(), kw.contiguous()
 
-    def forward(self, x: torch.Tensor, step, cache) -> torch.Tensor:
+    def forward(self, x, step, cache, fold=None):
         ops = self.ctx.ops
         qkv = self.qkv.forward(x)
         fused = self.position.fused_rotary(step)
@@ -108,4 +109,4 @@ class PagedAttention(Mixer):
             q, cache.kv, group.block_table, step.seq_slots, step.cu_tokens, step.kv_lens, step.token_seq,
             self.window, self.scale, step.min_q_len, step.max_q_len, step.max_kv_len,
         )
-        return self.o.forward(a)
+        return self.o.forward(a, fold=fold)

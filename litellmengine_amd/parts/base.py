@@ -56,13 +56,42 @@ class Part:
         self.ctx = ctx
 
 
+@dataclasses.dataclass
+class NormFold:
+    """A request to the product that precedes a norm: add your result into the 32-bit
+    residual stream `hidden` in place and hand on the norm's input as a `Prenormed`,
+    so that the norm needs no launch of its own."""
+
+    hidden: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+
+@dataclasses.dataclass
+class Prenormed:
+    """Normed rows whose last factor is still outstanding: row m of the norm's result is
+    `xw[m] * rsqrt(sum(sums[:, m]) / width + eps)`.  That factor commutes with a
+    product, so the product that follows applies it to its own result.  Only
+    `ops.linear` and `ops.gate_up_silu` take one, and each value is used once."""
+
+    xw: torch.Tensor  # [N, width], hidden * norm weight, activation type
+    sums: torch.Tensor  # float32 [parts, 16]: sums of squares of hidden over column ranges, by row
+    eps: float
+
+
 class Norm(Part):
     """forward(hidden, delta) adds `delta` (or nothing) into the 32-bit residual
     stream `hidden` in place and returns the normed rows in the activation type;
-    with `rows` only those rows are read and `hidden` is left alone."""
+    with `rows` only those rows are read and `hidden` is left alone.
+
+    fold(hidden) may return a NormFold when the step is small enough that the
+    products on both sides of the norm can do its work (None: call forward)."""
 
     def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], rows=None) -> torch.Tensor:
         raise NotImplementedError
+
+    def fold(self, hidden: torch.Tensor) -> Optional[NormFold]:
+        return None
 
 
 class PositionEncoding(Part):
@@ -91,6 +120,9 @@ class Mixer(Part):
     # the batch, no sizes that depend on the step's values): decode steps of such
     # mixers may be captured into a graph and replayed.
     graph_safe = False
+    # True if forward() takes a Prenormed for x (passing it to one product only) and
+    # a keyword `fold` (a NormFold for its last product, whose Prenormed it then returns).
+    folds_norm = False
 
     def cache_spec(self) -> Optional[KVCacheSpec]:
         return None
@@ -105,6 +137,8 @@ class Mixer(Part):
 class FeedForward(Part):
     """forward(x [N, hidden]) -> [N, hidden], token by token."""
 
+    folds_norm = False  # as Mixer.folds_norm
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
@@ -115,9 +149,16 @@ class Block(Part):
     forward(hidden, delta, step, cache) -> delta': `hidden` is the 32-bit
     residual stream [N, hidden]; `delta` is what the previous block still has to
     add to it (None for the first); the return value is what this block leaves
-    to be added by whoever comes next."""
+    to be added by whoever comes next.
+
+    A block whose first norm can be folded into the products around it says so
+    with entry_norm(); the model then passes the next block's as `next_norm`, and
+    the block may return a Prenormed made for that norm instead of a delta."""
 
     mixer: Mixer
 
-    def forward(self, hidden, delta, step, cache):
+    def entry_norm(self) -> Optional[Norm]:
+        return None
+
+    def forward(self, hidden, delta, step, cache, next_norm=None):
         raise NotImplementedError

@@ -6,7 +6,7 @@ from __future__ import annotations
 from typing import Dict
 
 from ..weights.spec import TensorSpec
-from .base import Block, BuildContext, FeedForward, Mixer, Norm
+from .base import Block, BuildContext, FeedForward, Mixer, Norm, Prenormed
 
 
 class PreNormBlock(Block):
@@ -30,8 +30,18 @@ class PreNormBlock(Block):
         for p in self._parts():
             p.bind(weights, ctx)
 
-    def forward(self, hidden, delta, step, cache):
-        x = self.norm_in.forward(hidden, delta)
-        a = self.mixer.forward(x, step, cache)
-        x = self.norm_post.forward(hidden, a)
+    def entry_norm(self):
+        return self.norm_in if self.mixer.folds_norm else None
+
+    def forward(self, hidden, delta, step, cache, next_norm=None):
+        # a Prenormed was made for norm_in by the block before: the add and the norm are done
+        x = delta if isinstance(delta, Prenormed) else self.norm_in.forward(hidden, delta)
+        fold = self.norm_post.fold(hidden) if self.mixer.folds_norm and self.feed_forward.folds_norm else None
+        if fold is not None:
+            x = self.mixer.forward(x, step, cache, fold=fold)
+        else:
+            x = self.norm_post.forward(hidden, self.mixer.forward(x, step, cache))
+        fold = next_norm.fold(hidden) if next_norm is not None and self.feed_forward.folds_norm else None
+        if fold is not None:
+            return self.feed_forward.forward(x, fold=fold)
         return self.feed_forward.forward(x)

@@ -13,6 +13,8 @@ from .linear import Linear
 
 
 class GatedMLP(FeedForward):
+    folds_norm = True
+
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
         self.gate_up = Linear(
             [prefix + "gate_proj.weight", prefix + "up_proj.weight"], hidden_size, [intermediate_size] * 2
@@ -27,5 +29,5 @@ class GatedMLP(FeedForward):
         self.gate_up.bind(weights, ctx)
         self.down.bind(weights, ctx)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down.forward(self.ctx.ops.gate_up_silu(x, self.gate_up.weight))
+    def forward(self, x, fold=None):
+        return self.down.forward(self.ctx.ops.gate_up_silu(x, self.gate_up.weight), fold=fold)

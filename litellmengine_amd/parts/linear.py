@@ -36,5 +36,9 @@ class Linear(Part):
         self.ctx = ctx
         self.weight = tensor
 
-    def forward(self, x: torch.Tensor, out_dtype=None) -> torch.Tensor:
-        return self.ctx.ops.linear(x, self.weight, out_dtype)
+    def forward(self, x, out_dtype=None, fold=None):
+        """`x` may be a parts.base.Prenormed; with `fold` (a parts.base.NormFold) the result
+        is added into the residual stream and comes back as the Prenormed of that norm."""
+        if fold is None:
+            return self.ctx.ops.linear(x, self.weight, out_dtype)
+        return self.ctx.ops.linear(x, self.weight, out_dtype, fold=fold)

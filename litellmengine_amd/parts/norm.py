@@ -8,7 +8,7 @@ from typing import Dict, Optional
 import torch
 
 from ..weights.spec import INIT_NORM, TensorSpec
-from .base import BuildContext, Norm
+from .base import BuildContext, Norm, NormFold
 
 
 class RMSNorm(Norm):
@@ -27,3 +27,9 @@ class RMSNorm(Norm):
 
     def forward(self, hidden, delta, rows=None) -> torch.Tensor:
         return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)
+
+    def fold(self, hidden) -> Optional[NormFold]:
+        can = getattr(self.ctx.ops, "can_fold_norm", None)  # an ops object without it never folds
+        if can is None or not can(hidden.shape[0], self.size, self.ctx.dtype):
+            return None
+        return NormFold(hidden, self.weight, self.eps)

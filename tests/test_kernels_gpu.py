@@ -98,6 +98,51 @@ def test_gate_up_silu(dtype, M, I, K):
     assert (got.double() - want).abs().max() < lim * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M,H,K,N", [(1, 64, 40, 48), (3, 136, 72, 100), (8, 4096, 1024, 512), (5, 1000, 64, 30),
+                                     (7, 24, 8, 6)])
+def test_norm_folded_into_products(wdtype, M, H, K, N):
+    """RMSNorm between two products, done by them: the first adds its result into the
+    residual stream and leaves hidden * w and sums of squares, the second (plain or
+    gated) scales its rows.  Compared with add, norm, product in float64; the hidden row
+    is made large in one place so that a missing or doubled part of the sum shows."""
+    from litellmengine_amd.parts import NormFold
+
+    o = ops()
+    assert o.can_fold_norm(M, H, torch.bfloat16) and not o.can_fold_norm(9, H, torch.bfloat16)
+    assert not o.can_fold_norm(M, H, torch.float32) and not o.can_fold_norm(M, H + 4, torch.bfloat16)
+    a = rnd((M, K), torch.bfloat16, 31)
+    w1 = rnd((H, K), torch.bfloat16, 32, 0.2)
+    hidden = rnd((M, H), torch.float32, 33, 1.5)
+    hidden[:, H - 3] += 20.0  # a column of the last, partly filled, workgroup dominates the mean
+    nw = (1 + 0.3 * rnd((H,), torch.float32, 34)).to(wdtype)
+    eps = 1e-3
+    for gated in (False, True):
+        w2 = rnd((2 * N if gated else N, H), torch.bfloat16, 35, 0.1)
+        h = hidden.clone()
+        pre = o.linear(a, w1, fold=NormFold(h, nw, eps))
+        want_h = hidden.double() + a.double() @ w1.double().t()
+        assert (h.double() - want_h).abs().max() < 1e-4 * max(1.0, want_h.abs().max().item())
+        assert pre.sums.shape == ((H + 15) // 16, 16)
+        ss = pre.sums.double().sum(0)[:M]
+        assert torch.allclose(ss, (want_h ** 2).sum(1), rtol=1e-5)
+        normed = want_h * torch.rsqrt((want_h ** 2).mean(1, keepdim=True) + eps) * nw.double()
+        y = normed @ w2.double().t()
+        if gated:
+            got = o.gate_up_silu(pre, w2)
+            want = torch.nn.functional.silu(y[:, :N]) * y[:, N:]
+        else:
+            got = o.linear(pre, w2)
+            want = y
+        assert got.dtype == torch.bfloat16 and got.shape == want.shape
+        assert (got.double() - want).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+        # against the unfolded kernels on the same numbers: the two differ by rounding only
+        h2 = hidden.clone()
+        x2 = o.add_rmsnorm(h2, o.linear(a, w1), nw, eps, torch.bfloat16)
+        ref = o.gate_up_silu(x2, w2) if gated else o.linear(x2, w2)
+        assert (got.double() - ref.double()).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+
+
 def test_silu_mul_reference_vector():
     # tests/test_silu_and_mul.cpp:48-56
     g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])
