@@ -313,6 +313,29 @@ def _attention_fast(q, k, v, window):
     return torch.einsum("hts,shd->thd", p, v)
 
 
+def first_layer_attention_probs(ids, w, cfg) -> torch.Tensor:
+    """Softmax weights [nq, T, T] of the first layer (tests use it to see how peaked
+    the attention of a model is)."""
+    T = len(ids)
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    eps, theta = cfg["rms_norm_eps"], cfg["rope_theta"]
+    p = "model.layers.0."
+    h = w["model.embed_tokens.weight"][torch.tensor(list(ids), dtype=torch.long)]
+    x = rms_norm(h, w[p + "input_layernorm.weight"], eps)
+    q = fast_linear(x, w[p + "self_attn.q_proj.weight"]).reshape(T, nq, d)
+    k = fast_linear(x, w[p + "self_attn.k_proj.weight"]).reshape(T, nkv, d)
+    q = _rope_fast(rms_norm(q, w[p + "self_attn.q_norm.weight"], eps), range(T), theta)
+    k = _rope_fast(rms_norm(k, w[p + "self_attn.k_norm.weight"], eps), range(T), theta)
+    k = k.repeat_interleave(nq // nkv, dim=1)
+    scores = torch.einsum("thd,shd->hts", q, k) / math.sqrt(d)
+    t = torch.arange(T)
+    allowed = t[None, :] <= t[:, None]
+    window = layer_windows(cfg)[0]
+    if window is not None:
+        allowed = allowed & (t[None, :] > t[:, None] - window)
+    return torch.softmax(scores.masked_fill(~allowed[None], float("-inf")), dim=-1)
+
+
 def model_logits_fast(ids, w, cfg, positions=None) -> torch.Tensor:
     T = len(ids)
     positions = list(range(T)) if positions is None else positions

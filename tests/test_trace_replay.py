@@ -6,7 +6,7 @@ bfloat16; the CPU test runs its main() with substitute kernels."""
 import pytest
 import torch
 
-from tests.tiny import CONFIGS, PAGE_SIZES, make_model_dir, random_tokens
+from tests.tiny import CONFIGS, PAGE_SIZES, make_model_dir, random_tokens, sharpen_attention
 from tests.torch_ops import TorchOps
 from tests.trace_util import (TraceBuilder, changing_portions, check_dumps, mixed, plain_logits, run_tool,
                               tail_one_by_one, whole)
@@ -51,3 +51,59 @@ def test_trace_gpu(tmp_path, which, dtype):
     run_tool(d, dtype, out, tb, page_size=PAGE_SIZES[which] if which != "A" else None)
     worst = check_dumps(out, tb, plain_logits(d, requests), TOL[dtype])
     print(f"trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
+
+
+def peaked_trace(vocab):
+    """Long requests (a far key among hundreds) in every way of cutting, few pages."""
+    requests = {"p": random_tokens(300, vocab, 41), "q": random_tokens(170, vocab, 42),
+                "r": random_tokens(230, vocab, 43), "s": random_tokens(90, vocab, 44)}
+    tb = TraceBuilder()
+    whole(tb, "p#whole", requests["p"])
+    tail_one_by_one(tb, "p#tail", requests["p"])
+    changing_portions(tb, "r#cut", requests["r"], seed=3)
+    mixed(tb, {rid + "#mix": t for rid, t in requests.items()}, seed=6)
+    return requests, tb
+
+
+# Larger scores carry the rounding of q and k further into the softmax weights: with the
+# factors below, a float32 run of plain torch on the CPU (tests/torch_ops.py, no code shared
+# with the kernels) is up to 5e-5 from the float64 model, a bfloat16 run up to 5e-2.  One key
+# lost at a window's edge moves the logits of these models by 0.35 (median over positions).
+PEAK = {"float32": (3.0, 1e-4), "bfloat16": (2.0, 1e-1)}
+
+
+def attention_is_peaked(model_dir, tokens, share):
+    """The plain model's first layer gives one key more than half of the weight for
+    at least `share` of the queries past the first few: the sharpening did what it is for."""
+    from tests.plain import qwen3_plain as plain
+
+    cfg, w = plain.read_model_dir(model_dir)
+    probs = plain.first_layer_attention_probs(tokens, w, cfg)  # [heads, T, T]
+    top = probs[:, 32:, :].max(dim=-1).values
+    return (top > 0.5).double().mean().item() > share
+
+
+def test_peaked_attention_trace_cpu(tmp_path):
+    d = make_model_dir(tmp_path, "C")
+    factor, tol = PEAK["float32"]
+    sharpen_attention(d, factor)
+    requests, tb = peaked_trace(CONFIGS["C"]["vocab_size"])
+    assert attention_is_peaked(d, requests["p"], 0.8)
+    out = str(tmp_path / "out")
+    run_tool(d, "float32", out, tb, in_process_ops=TorchOps())
+    check_dumps(out, tb, plain_logits(d, requests), tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["B", "C"])
+def test_peaked_attention_trace_gpu(tmp_path, which, dtype):
+    d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
+    factor, tol = PEAK[dtype]
+    sharpen_attention(d, factor)
+    requests, tb = peaked_trace(CONFIGS[which]["vocab_size"])
+    assert attention_is_peaked(d, requests["p"], 0.35)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=PAGE_SIZES[which])
+    worst = check_dumps(out, tb, plain_logits(d, requests), tol)
+    print(f"peaked trace {which} {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")

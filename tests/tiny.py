@@ -39,6 +39,21 @@ def make_model_dir(tmp_path, which: str, seed: int = 1234, dtype=torch.float32) 
     return path
 
 
+def sharpen_attention(model_dir: str, factor: float) -> None:
+    """Multiply the q and k norm weights of a model folder by `factor`: scores grow by
+    factor^2, so every query picks out one or two keys, near or far, instead of averaging
+    all of them.  A key that is lost, doubled or read from the wrong page then moves the
+    logits by far more than rounding does."""
+    from safetensors.torch import load_file, save_file
+
+    path = os.path.join(model_dir, "model.safetensors")
+    tensors = load_file(path)
+    for name in tensors:
+        if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
+            tensors[name] = (tensors[name].float() * factor).to(tensors[name].dtype)
+    save_file(tensors, path, metadata={"format": "pt"})
+
+
 def random_tokens(n: int, vocab: int, seed: int):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
