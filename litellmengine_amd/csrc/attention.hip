@@ -190,6 +190,13 @@ __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&
         st.open_lo[t] = lo_max;
         st.open_hi[t] = pos_min == 0x7fffffff ? -1 : pos_min;
     }
+    // The rows of Q are waited for here, once.  Left pending, their first use lies inside the
+    // key loop, where the wait for them also waits for the K/V loads just issued for a later
+    // step: the loop would run at the latency of memory.
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) asm volatile("" : "+v"(st.qv[t][ks]));
 }
 
 // One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key r16 of
@@ -211,6 +218,12 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
             for (int t = 0; t < RT; ++t)
                 s[t][x] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k, st.qv[t][ks], s[t][x], 0, 0, 0);
         }
+    // the value operands are asked for before the softmax, whose arithmetic covers their way
+    // from LDS; asked for one by one between the products, each would be waited for in turn
+    bf16x8 vv[2 * DK];
+#pragma unroll
+    for (int n = 0; n < 2 * DK; ++n) vv[n] = load_v(n);
+    __builtin_amdgcn_sched_barrier(0);
     bf16x8 pb[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
@@ -250,9 +263,9 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
     }
 #pragma unroll
     for (int n = 0; n < 2 * DK; ++n) {
-        const bf16x8 v = load_v(n);
 #pragma unroll
-        for (int t = 0; t < RT; ++t) st.o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pb[t], st.o[t][n], 0, 0, 0);
+        for (int t = 0; t < RT; ++t)
+            st.o[t][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv[n], pb[t], st.o[t][n], 0, 0, 0);
     }
 }
 
@@ -266,8 +279,20 @@ __device__ __forceinline__ void finish_rows(RowState<DK, RT>& st) {
     }
 }
 
+// The operands of one 32-key step as a wavefront loads them straight from the pages.
+template <int DK>
+struct StepOperands {
+    bf16x8 k[2][DK];
+    bf16x4 v[2 * DK][2];
+};
+
 // The steps step_begin, step_begin + step_stride, ... < step_end with the operands loaded by
-// each wavefront straight from the pages.
+// each wavefront straight from the pages, two steps ahead of their use: while one step is
+// multiplied the loads of the next two are on their way.  Nothing in the loop stands under a
+// condition (a load under a condition makes the compiler wait for every load where the paths
+// meet again): the loop runs an even number of steps, loads past the end go to a page that is
+// there, and the CALLER has limited the rows' `pos` to the last key of step_end - 1, so that a
+// step past the end is masked out whole.
 template <int DK, int RT>
 __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT],
                                             const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ table,
@@ -277,35 +302,59 @@ __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo 
     const int lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
     init_rows<DK, RT>(st, row);
-    const int64_t k_head = (int64_t)kvh * P * D;
-    const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
-    for (int step = step_begin; step < step_end; step += step_stride) {
-        const int j0 = step * KSTEP;
-        const bf16_t* page[2];
-        int off[2];
+    const int64_t k_lane = (int64_t)kvh * P * D + (int64_t)r16 * D + 8 * c;
+    const int64_t v_lane = ((int64_t)nkv + kvh) * P * D + (int64_t)r16 * P + 4 * c;
+    // Page and offset of a step's first key are carried from step to step instead of divided
+    // out each time (the page size is no constant), and the table is read one load ahead.  A
+    // half wholly outside [lo_min, hi] may lie in a page that is not there: the page index is
+    // clamped to those of keys that are.
+    const int page_lo = lo_min / P, page_hi = hi / P;
+    const int adv_pages = (step_stride * KSTEP) / P, adv_off = (step_stride * KSTEP) % P;
+    int look_page = (step_begin * KSTEP) / P, look_off = (step_begin * KSTEP) % P;
+    int page_id[2], page_off[2];
+    auto lookup = [&]() {
+        const bool next_page = look_off + 16 == P;  // pages hold a multiple of 16 keys
+        const int pg[2] = {look_page, next_page ? look_page + 1 : look_page};
+        page_off[0] = look_off;
+        page_off[1] = next_page ? 0 : look_off + 16;
+#pragma unroll
+        for (int x = 0; x < 2; ++x)  // the same for the whole wavefront: a scalar load, which no vector load waits for
+            page_id[x] = table[__builtin_amdgcn_readfirstlane(min(max(pg[x], page_lo), page_hi))];
+        look_page += adv_pages;
+        look_off += adv_off;
+        if (look_off >= P) {
+            look_off -= P;
+            ++look_page;
+        }
+    };
+    auto load = [&](StepOperands<DK>& op) {
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
-            const int jx = j0 + 16 * x;
-            // a tile wholly outside [lo_min, hi] may lie in a page that is not there: look up a key that is
-            const int probe = min(max(jx, lo_min), hi);
-            page[x] = kv_layer + (int64_t)table[probe / P] * page_stride;
-            off[x] = jx % P;
+            const bf16_t* page = kv_layer + (int64_t)page_id[x] * page_stride;
+            const bf16_t* kp = page + k_lane + (int64_t)page_off[x] * D;
+            const bf16_t* vp = page + v_lane + page_off[x];
+#pragma unroll
+            for (int ks = 0; ks < DK; ++ks) op.k[x][ks] = *(const bf16x8*)(kp + 32 * ks);
+#pragma unroll
+            for (int n = 0; n < 2 * DK; ++n) op.v[n][x] = *(const bf16x4*)(vp + (int64_t)16 * n * P);
         }
-        bf16x8 ka[2][DK];
-#pragma unroll
-        for (int x = 0; x < 2; ++x)
-#pragma unroll
-            for (int ks = 0; ks < DK; ++ks)
-                ka[x][ks] = *(const bf16x8*)(page[x] + k_head + (int64_t)(off[x] + r16) * D + 32 * ks + 8 * c);
-        bf16x4 va[2 * DK][2];
-#pragma unroll
-        for (int n = 0; n < 2 * DK; ++n)
-#pragma unroll
-            for (int x = 0; x < 2; ++x)
-                va[n][x] = *(const bf16x4*)(page[x] + v_head + (int64_t)(16 * n + r16) * P + off[x] + 4 * c);
+        lookup();
+    };
+    auto multiply = [&](const StepOperands<DK>& op, int step) {
         tile_step<DK, RT>(
-            st, row, [&](int x, int ks) { return ka[x][ks]; },
-            [&](int n) { return __builtin_shufflevector(va[n][0], va[n][1], 0, 1, 2, 3, 4, 5, 6, 7); }, j0, scale_log2);
+            st, row, [&](int x, int ks) { return op.k[x][ks]; },
+            [&](int n) { return __builtin_shufflevector(op.v[n][0], op.v[n][1], 0, 1, 2, 3, 4, 5, 6, 7); },
+            step * KSTEP, scale_log2);
+    };
+    StepOperands<DK> even, odd;
+    lookup();
+    load(even);
+    load(odd);
+    for (int step = step_begin; step < step_end; step += 2 * step_stride) {
+        multiply(even, step);
+        load(even);
+        multiply(odd, step + step_stride);
+        load(odd);
     }
     finish_rows<DK, RT>(st);
 }
@@ -364,6 +413,8 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int per_split = (last - first + 1 + nsplit - 1) / nsplit;
     const int sb = first + split * per_split;
     const int se = min(last + 1, sb + per_split);
+    // keys of later splits are not this workgroup's: attend_rows may run a step past `se`
+    row[0].pos = min(row[0].pos, se * KSTEP - 1);
 
     RowState<DK, 1> st;
     attend_rows<DK, 1>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi,
@@ -472,16 +523,18 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     constexpr int TILE = KSTEP * KROW + D * VROW;
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * TILE];
 
-    const int s = blockIdx.z, kvh = blockIdx.y;
+    // the kv head varies fastest: workgroups go to the eight dies in turn, each die has an L2 of
+    // its own, and this way a die sees the K/V of few heads, which the row blocks of a head share
+    const int s = blockIdx.z, kvh = blockIdx.x;
     const int G = nq / nkv;
     const int q_start = cu_tokens[s];
     const int q_len = cu_tokens[s + 1] - q_start;
     const int nrows = q_len * G;
     if (nrows <= 16) return;  // the decode kernel's
     // the last rows see the most keys: they are started first
-    const int row_blocks = gridDim.x / nsplit;
-    const int split = blockIdx.x / row_blocks;
-    const int block_row0 = (row_blocks - 1 - blockIdx.x % row_blocks) * PRE_ROWS;
+    const int row_blocks = gridDim.y / nsplit;
+    const int split = blockIdx.y / row_blocks;
+    const int block_row0 = (row_blocks - 1 - blockIdx.y % row_blocks) * PRE_ROWS;
     if (block_row0 >= nrows) return;
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
@@ -510,7 +563,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
         const int my_last_row = min(nrows, row0 + 16 * PRE_RT) - 1;
         const int my_lo = window > 0 ? max(0, past + row0 / G - window + 1) : 0;
         my_first = my_lo / KSTEP;
-        my_end = (past + my_last_row / G) / KSTEP + 1;
+        my_end = min(end_step, (past + my_last_row / G) / KSTEP + 1);
     }
     RowState<DK, PRE_RT> st;
     init_rows<DK, PRE_RT>(st, row);
@@ -523,17 +576,35 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     // two tiles are on their way from memory at any time (register sets 0 and 1); a tile is
     // written to LDS one step after its loads were issued and multiplied one step later still
     bf16x8 stage_k[2][NP], stage_v[2][NP];
-    auto fetch = [&](int step, auto set_c) {
+    // The pages of the two 16-key halves of a step are looked up one fetch ahead, so that the
+    // table's latency is not in the way of the loads that need it.  Fetches come in step order:
+    // page and offset of the next half are carried along instead of divided out (the page size
+    // is no constant).  A half wholly outside [lo_min, hi] may lie in a page that is not there:
+    // the page index is clamped to those of keys that are.
+    const int page_lo = lo_min / P, page_hi = hi / P;
+    int look_page = (first_step * KSTEP) / P, look_off = (first_step * KSTEP) % P;
+    int page_id[2], page_off[2];
+    auto lookup = [&]() {
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            page_id[x] = table[__builtin_amdgcn_readfirstlane(min(max(look_page, page_lo), page_hi))];
+            page_off[x] = look_off;
+            look_off += 16;  // pages hold a multiple of 16 keys
+            if (look_off == P) {
+                look_off = 0;
+                ++look_page;
+            }
+        }
+    };
+    lookup();
+    auto fetch = [&](auto set_c) {
         constexpr int set = decltype(set_c)::value;
-        const int j0 = step * KSTEP;
         const bf16_t* page[2];
         int off[2];
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
-            const int jx = j0 + 16 * x;
-            const int probe = min(max(jx, lo_min), hi);
-            page[x] = kv_layer + (int64_t)table[probe / P] * page_stride;
-            off[x] = jx % P;
+            page[x] = kv_layer + (int64_t)page_id[x] * page_stride;
+            off[x] = page_off[x];
         }
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
@@ -549,6 +620,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
                                                    (xv ? off[1] : off[0]) + (part % 2) * 8);
             }
         }
+        lookup();
     };
     auto stash = [&](int buf, auto set_c) {
         constexpr int set = decltype(set_c)::value;
@@ -570,9 +642,12 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     // one step: tile `step` is in LDS buffer `buf`; tile step + 1 sits in register set `set`
     // (loads issued a step ago) and goes to the other buffer; tile step + 2 is requested now
     // into the other register set
+    // Fetch and stash run in every step, also past the last tile (the lookup clamps to a page
+    // that is there; what is stashed then is never read): a load under a condition makes the
+    // compiler wait, where the paths meet again, for the loads that were issued last.
     auto one_step = [&](int step, int buf, auto set_c) {
         constexpr int set = decltype(set_c)::value;
-        if (step + 2 < end_step) fetch(step + 2, std::integral_constant<int, 1 - set>{});
+        fetch(std::integral_constant<int, 1 - set>{});  // tile step + 2
         if (step >= my_first && step < my_end) {
             const bf16_t* kt = lds + buf * TILE;
             const bf16_t* vt = kt + KSTEP * KROW;
@@ -584,19 +659,17 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
                 },
                 step * KSTEP, scale_log2);
         }
-        if (step + 1 < end_step) stash(buf ^ 1, set_c);
+        stash(buf ^ 1, set_c);
         __syncthreads();
     };
 
-    if (first_step < end_step) {
-        fetch(first_step, std::integral_constant<int, 0>{});
-        if (first_step + 1 < end_step) fetch(first_step + 1, std::integral_constant<int, 1>{});
-        stash(0, std::integral_constant<int, 0>{});
-    }
+    fetch(std::integral_constant<int, 0>{});  // tile first_step
+    fetch(std::integral_constant<int, 1>{});  // tile first_step + 1
+    stash(0, std::integral_constant<int, 0>{});
     __syncthreads();
     for (int step = first_step; step < end_step; step += 2) {
         one_step(step, 0, std::integral_constant<int, 1>{});
-        if (step + 1 < end_step) one_step(step + 1, 1, std::integral_constant<int, 0>{});
+        one_step(step + 1, 1, std::integral_constant<int, 0>{});  // multiplies nothing past my_end
     }
     finish_rows<DK, PRE_RT>(st);
 #pragma unroll
@@ -654,7 +727,7 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
         constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT_OF(DK);
         const int rows = max_q_len * G;
         const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
-        mfma_prefill_kernel<DK><<<dim3(blocks * nsplit_prefill, nkv, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
+        mfma_prefill_kernel<DK><<<dim3(nkv, blocks * nsplit_prefill, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
             q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill, nq,
             nkv, P, page_stride, max_pages, window, scale_log2);
     }
