@@ -137,6 +137,7 @@ typedef bf16_t bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define NEG_BIG (-1.0e30f)
+#define LAZY_MAX 8.0f  // a row's reference maximum may lag its true one by this much (base 2)
 #define KSTEP 32  // keys per step: two 16-key tiles, each inside one page
 
 // What one lane knows about the query row it serves (row = lane % 16 of a 16-row tile).
@@ -224,42 +225,64 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
 #pragma unroll
     for (int n = 0; n < 2 * DK; ++n) vv[n] = load_v(n);
     __builtin_amdgcn_sched_barrier(0);
-    bf16x8 pb[RT];
+    // Scores relative to the row's reference m, in the base-2 domain: x = s * scale - m.  The
+    // reference only has to be near the row's maximum, not equal to it: while no x exceeds
+    // LAZY_MAX the weights are exp2(x) <= 2^LAZY_MAX and nothing else is touched.  Only when
+    // some row of the wavefront goes beyond (the first keys of a row always do: m starts at
+    // NEG_BIG) the maxima are agreed on between the four lanes of each row and m, l and the
+    // accumulators are moved; that is rare after a row's first steps.
+    float x[RT][8];
+    bool raise = false;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-        // scores of row r16 for keys j0 + 16 x + 4 c + i, in the base-2 domain
-        float sc[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) sc[i] = s[t][i / 4][i % 4] * scale_log2;
+        for (int i = 0; i < 8; ++i) x[t][i] = fmaf(s[t][i / 4][i % 4], scale_log2, -st.m[t]);
         if (!(j0 >= st.open_lo[t] && j0 + KSTEP - 1 <= st.open_hi[t])) {  // same for the whole wavefront
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int j = j0 + 16 * (i / 4) + 4 * c + (i % 4);
-                if (j < row[t].lo || j > row[t].pos) sc[i] = NEG_BIG;
+                if (j < row[t].lo || j > row[t].pos) x[t][i] = NEG_BIG;
             }
         }
-        float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                               fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
-        const float new_m = fmaxf(st.m[t], tile_max);
-        // a masked score is NEG_BIG; while the row has seen no key yet new_m is NEG_BIG too,
-        // and exp2(0) = 1 would count the masked key: shift such rows so that they give 0
-        const float base = new_m <= NEG_BIG ? 0.f : new_m;
-        const float alpha = __builtin_amdgcn_exp2f(st.m[t] - base);
-        st.m[t] = new_m;
+        const float top = fmaxf(fmaxf(fmaxf(x[t][0], x[t][1]), fmaxf(x[t][2], x[t][3])),
+                                fmaxf(fmaxf(x[t][4], x[t][5]), fmaxf(x[t][6], x[t][7])));
+        raise = raise || top > LAZY_MAX;
+    }
+    if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            // absolute scores again (x has lost them where m was still NEG_BIG)
+            float sc[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] = x[t][i] <= NEG_BIG ? NEG_BIG : s[t][i / 4][i % 4] * scale_log2;
+            float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                                   fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
+            const float new_m = fmaxf(st.m[t], tile_max);
+            // while the row has seen no key new_m is NEG_BIG as its masked scores are, and
+            // exp2(0) = 1 would count them: shift such rows so that they give 0
+            const float base = new_m <= NEG_BIG ? 0.f : new_m;
+            const float alpha = __builtin_amdgcn_exp2f(st.m[t] - base);
+            st.m[t] = new_m;
+            st.l[t] *= alpha;
+#pragma unroll
+            for (int n = 0; n < 2 * DK; ++n) st.o[t][n] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[t][i] = sc[i] - base;
+        }
+    }
+    bf16x8 pb[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
         float psum = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float p = __builtin_amdgcn_exp2f(sc[i] - base);
+            const float p = __builtin_amdgcn_exp2f(x[t][i]);
             psum += p;
             pb[t][i] = (bf16_t)p;
         }
-        st.l[t] = st.l[t] * alpha + psum;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum moved somewhere
-#pragma unroll
-            for (int n = 0; n < 2 * DK; ++n) st.o[t][n] *= alpha;
-        }
+        st.l[t] += psum;
     }
 #pragma unroll
     for (int n = 0; n < 2 * DK; ++n) {
@@ -573,6 +596,8 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     // a tile holds 4 D 16-byte pieces of K and as many of V^T; this thread copies NP of each
     constexpr int PIECES = 4 * D;
     constexpr int NP = (PIECES + PRE_WAVES * LLE_WAVE - 1) / (PRE_WAVES * LLE_WAVE);
+    // then the copies stand under no condition (see one_step on what a condition costs)
+    constexpr bool EVERY_THREAD_COPIES = PIECES % (PRE_WAVES * LLE_WAVE) == 0;
     // two tiles are on their way from memory at any time (register sets 0 and 1); a tile is
     // written to LDS one step after its loads were issued and multiplied one step later still
     bf16x8 stage_k[2][NP], stage_v[2][NP];
@@ -597,43 +622,46 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
         }
     };
     lookup();
+    // Piece `piece` of a tile: the wavefront-sized run it lies in belongs to ONE 16-key half
+    // (half = run / DK), so the half's page is the same for the whole wavefront and its address
+    // stays in scalar registers; what differs between the threads is fixed for the kernel.
+    //   K: the half's keys row by row, 16 bytes of a row per piece;
+    //   V^T: the half's value elements one by one, each 16 keys = two pieces.
+    int k_thread[NP], v_thread[NP];  // element offsets from the half's first key, in the page
+    int k_lds[NP], v_lds[NP];        // element offsets in a tile in LDS
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int q = (threadIdx.x + PRE_WAVES * LLE_WAVE * i) % (2 * D);  // piece within its half
+        const int half = (threadIdx.x + PRE_WAVES * LLE_WAVE * i) / (2 * D);
+        k_thread[i] = (q / (D / 8)) * D + (q % (D / 8)) * 8;
+        v_thread[i] = (q / 2) * P + (q % 2) * 8;
+        k_lds[i] = (16 * half + q / (D / 8)) * KROW + (q % (D / 8)) * 8;
+        v_lds[i] = KSTEP * KROW + (q / 2) * VROW + 16 * half + (q % 2) * 8;
+    }
     auto fetch = [&](auto set_c) {
         constexpr int set = decltype(set_c)::value;
-        const bf16_t* page[2];
-        int off[2];
-#pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            page[x] = kv_layer + (int64_t)page_id[x] * page_stride;
-            off[x] = page_off[x];
-        }
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int piece = threadIdx.x + PRE_WAVES * LLE_WAVE * i;
-            if (piece < PIECES) {
-                const int key = piece / (D / 8), ch = piece % (D / 8);  // key 0..31, 16-byte piece of its row
-                const int xk = key / 16;
-                stage_k[set][i] = *(const bf16x8*)((xk ? page[1] : page[0]) + k_head +
-                                                   (int64_t)((xk ? off[1] : off[0]) + key % 16) * D + ch * 8);
-                const int dd = piece / 4, part = piece % 4;  // value element 0..D-1, quarter of its 32 keys
-                const int xv = part / 2;
-                stage_v[set][i] = *(const bf16x8*)((xv ? page[1] : page[0]) + v_head + (int64_t)dd * P +
-                                                   (xv ? off[1] : off[0]) + (part % 2) * 8);
+            if (EVERY_THREAD_COPIES || piece < PIECES) {
+                const int half = __builtin_amdgcn_readfirstlane(piece / (2 * D));
+                const bf16_t* page = kv_layer + (int64_t)(half ? page_id[1] : page_id[0]) * page_stride;
+                const int off = half ? page_off[1] : page_off[0];
+                stage_k[set][i] = *(const bf16x8*)(page + k_head + (int64_t)off * D + k_thread[i]);
+                stage_v[set][i] = *(const bf16x8*)(page + v_head + off + v_thread[i]);
             }
         }
         lookup();
     };
     auto stash = [&](int buf, auto set_c) {
         constexpr int set = decltype(set_c)::value;
-        bf16_t* kt = lds + buf * TILE;
-        bf16_t* vt = kt + KSTEP * KROW;
+        bf16_t* tile = lds + buf * TILE;
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int piece = threadIdx.x + PRE_WAVES * LLE_WAVE * i;
-            if (piece < PIECES) {
-                const int key = piece / (D / 8), ch = piece % (D / 8);
-                *(bf16x8*)(kt + key * KROW + ch * 8) = stage_k[set][i];
-                const int dd = piece / 4, part = piece % 4;
-                bf16_t* dst = vt + dd * VROW + (part / 2) * 16 + (part % 2) * 8;  // 8-byte aligned
+            if (EVERY_THREAD_COPIES || piece < PIECES) {
+                *(bf16x8*)(tile + k_lds[i]) = stage_k[set][i];
+                bf16_t* dst = tile + v_lds[i];  // 8-byte aligned
                 *(bf16x4*)dst = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 0, 1, 2, 3);
                 *(bf16x4*)(dst + 4) = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 4, 5, 6, 7);
             }

@@ -135,6 +135,17 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
     const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
+    // RESID: thread (m, n) of the first 256 owns element [m][n0 + n]; what it needs of the
+    // residual stream and of the norm weight is asked for now and has arrived by the epilogue
+    float resid_h = 0.f, resid_w = 0.f;
+    if (RESID && threadIdx.x < 256) {
+        const int m = threadIdx.x / 16;
+        const int64_t col = n0 + threadIdx.x % 16;
+        if (m < M && col < N) {
+            resid_h = fold.hidden[(int64_t)m * N + col];
+            resid_w = load_as_f32(fold.weight, col, fold.weight_dtype);
+        }
+    }
     const bf16_t* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -233,7 +244,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
         }
         return;
     }
-    if (RESID) {  // NT = MT = 1: thread (m, n) of the first 256 owns element [m][n0 + n]
+    if (RESID) {  // NT = MT = 1
         if (threadIdx.x < 256) {
             const int m = threadIdx.x / 16, n = threadIdx.x % 16;
             const int64_t col = n0 + n;
@@ -242,9 +253,9 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
                 float sum = 0.f;
 #pragma unroll
                 for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][0][n][m];
-                const float h = fold.hidden[(int64_t)m * N + col] + sum;
+                const float h = resid_h + sum;
                 fold.hidden[(int64_t)m * N + col] = h;
-                fold.xw[(int64_t)m * N + col] = (bf16_t)(h * load_as_f32(fold.weight, col, fold.weight_dtype));
+                fold.xw[(int64_t)m * N + col] = (bf16_t)(h * resid_w);
                 sq = h * h;
             }
 #pragma unroll
