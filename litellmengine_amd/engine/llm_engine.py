@@ -32,12 +32,27 @@ class LLMEngine:
         self.verbose = verbose
         self.num_steps = 0
 
-    def add_request(self, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_id: int = -1,
-                    temperature: float = 0.0, seed: int = 0) -> Request:
-        for t in prompt_ids:
+    def _check_ids(self, token_ids: Sequence[int]) -> None:
+        for t in token_ids:
             if not 0 <= int(t) < self.model.vocab_size:
                 raise ValueError(f"token id {t} outside [0, {self.model.vocab_size})")
-        return self.scheduler.add_request(prompt_ids, max_new_tokens, eos_token_id, temperature, seed)
+
+    def add_request(self, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_id: int = -1,
+                    temperature: float = 0.0, seed: int = 0, keep_session: bool = False) -> Request:
+        """`keep_session`: the request keeps its cache when it finishes, for
+        append_input_tokens; release_request ends it."""
+        self._check_ids(prompt_ids)
+        return self.scheduler.add_request(prompt_ids, max_new_tokens, eos_token_id, temperature, seed, keep_session)
+
+    def append_input_tokens(self, request: Request, token_ids: Sequence[int], max_new_tokens: int,
+                            eos_token_id: int = -1) -> Request:
+        """A further turn of a finished request: its history, then `token_ids`, then up to
+        `max_new_tokens` new ones (src/engine/paged_generate_engine.cpp:81-97)."""
+        self._check_ids(token_ids)
+        return self.scheduler.append_input_tokens(request.request_id, token_ids, max_new_tokens, eos_token_id)
+
+    def release_request(self, request: Request) -> None:
+        self.scheduler.release_request(request.request_id)
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()

@@ -37,6 +37,10 @@ class Request:
     status: RequestStatus = RequestStatus.WAITING
     admitted_at: int = -1  # order of admission; the youngest is preempted first
     preemptions: int = 0
+    # a session: when it finishes it keeps its slot and pages, so that more input can be
+    # appended and only the new tokens are run (finishing does not free in the reference,
+    # src/engine/paged_generate_engine.cpp:386-395)
+    keep_session: bool = False
 
     def __post_init__(self):
         # a stream of its own: what a request draws does not depend on its batch mates
@@ -64,6 +68,19 @@ class Request:
         if num_tokens < 0 or self.cached_len + num_tokens > len(self.tokens):
             raise ValueError("mark_forward_done exceeds the request's tokens")
         self.cached_len += num_tokens
+
+    def append_input_tokens(self, token_ids, max_new_tokens: int, eos_token_id: int) -> None:
+        """A further turn: the history stays, the new tokens follow it, and what was
+        generated before no longer counts against max_new_tokens
+        (src/engine/request_manager.cpp:222-247, :256-279).  `cached_len` is left as
+        it is: the new tokens reach the cache in the next steps."""
+        if max_new_tokens < 0:
+            raise ValueError("max_new_tokens must be >= 0")
+        self.tokens.extend(int(t) for t in token_ids)
+        self.generated = []
+        self.prompt_len = len(self.tokens)
+        self.max_new_tokens = max_new_tokens
+        self.eos_token_id = int(eos_token_id)
 
     def append_token(self, token: int) -> None:
         """src/engine/request_manager.cpp:124-158"""

@@ -19,7 +19,14 @@ Here, every step:
     the pages for their first portion are there.
 A request that could never fit (its last cached position needs more pages than
 a group has, or than a request may hold) is refused when it is added.  Finished
-requests give their pages back at once.
+requests give their pages back at once, unless they were added as a session
+(`keep_session`): a finished session is PARKED with its slot and pages until
+`append_input_tokens` continues it (only the new tokens are run then, in
+portions like any prompt; the reference feeds them one by one,
+src/engine/paged_generate_engine.cpp:133-141) or `release_request` ends it.
+Parked sessions come before running requests when pages run out: the one
+parked longest loses its cache first (it is recomputed whole if it is ever
+continued).
 """
 from __future__ import annotations
 
@@ -54,13 +61,15 @@ class Scheduler:
         self.waiting: Deque[Request] = collections.deque()
         self.running: List[Request] = []
         self.requests: Dict[int, Request] = {}
+        self.parked: List[Request] = []  # finished sessions that still hold their cache, oldest first
         self._next_id = 0
         self._admissions = 0
         self.num_preemptions = 0
+        self.num_evictions = 0  # parked sessions whose cache was taken
 
     # -- adding ---------------------------------------------------------------------
     def add_request(self, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_id: int = -1,
-                    temperature: float = 0.0, seed: int = 0) -> Request:
+                    temperature: float = 0.0, seed: int = 0, keep_session: bool = False) -> Request:
         """src/engine/paged_generate_engine.cpp:57-79: a prompt must not be empty,
         max_new_tokens >= 0; 0 finishes at once."""
         if len(prompt_ids) == 0:
@@ -69,27 +78,82 @@ class Scheduler:
             raise ValueError("max_new_tokens must be >= 0")
         if temperature < 0:
             raise ValueError("temperature must be >= 0")
+        self._check_fits(len(prompt_ids), max_new_tokens)
         req = Request(self._next_id, [int(t) for t in prompt_ids], len(prompt_ids), max_new_tokens,
-                      int(eos_token_id), float(temperature), int(seed))
+                      int(eos_token_id), float(temperature), int(seed), keep_session=bool(keep_session))
         self._next_id += 1
         self.requests[req.request_id] = req
         if max_new_tokens == 0:
             req.status = RequestStatus.FINISHED
             return req
-        longest = req.prompt_len + max_new_tokens - 1  # the last token drawn is never cached
+        self.waiting.append(req)
+        return req
+
+    def _check_fits(self, prompt_len: int, max_new_tokens: int) -> None:
+        longest = prompt_len + max_new_tokens - 1  # the last token drawn is never cached
         for group in self.cache.groups:
             pages = group.pages_for(longest)
             if group.window is None and pages > group.pool.num_pages:
                 raise ValueError(
-                    f"request of {req.prompt_len} prompt + {max_new_tokens} new tokens needs {pages} pages, "
+                    f"request of {prompt_len} prompt + {max_new_tokens} new tokens needs {pages} pages, "
                     f"the cache has {group.pool.num_pages}"
                 )
             if pages > group.max_pages_per_request:
                 raise ValueError(
                     f"request needs {pages} pages, a request may hold {group.max_pages_per_request}"
                 )
-        self.waiting.append(req)
-        return req
+
+    def append_input_tokens(self, request_id: int, token_ids: Sequence[int], max_new_tokens: int,
+                            eos_token_id: int = -1) -> Request:
+        """Continue a finished request with more input (PagedGenerateEngine::append_input_tokens,
+        src/engine/paged_generate_engine.cpp:81-97).  A parked session runs on from its cache;
+        a request whose cache is gone waits to be recomputed from its first token."""
+        r = self.requests[request_id]
+        if not r.finished:
+            raise RuntimeError("append_input_tokens expects a finished request")
+        if max_new_tokens < 0:
+            raise ValueError("max_new_tokens must be >= 0")
+        self._check_fits(len(r.tokens) + len(token_ids), max_new_tokens)
+        r.append_input_tokens(token_ids, max_new_tokens, eos_token_id)
+        if max_new_tokens == 0 or r.extend_len == 0:
+            return r  # nothing to run: it stays finished (and parked, if it was)
+        if r in self.parked:
+            self.parked.remove(r)
+            r.status = RequestStatus.RUNNING
+            self.running.append(r)
+        else:
+            r.cached_len = 0
+            r.status = RequestStatus.WAITING
+            self.waiting.append(r)
+        return r
+
+    def release_request(self, request_id: int) -> None:
+        """Give back whatever the request still holds and end it
+        (PagedGenerateEngine::release_request, src/engine/paged_generate_engine.cpp:386-395)."""
+        r = self.requests[request_id]
+        if r in self.parked:
+            self.parked.remove(r)
+        if r in self.running:
+            self.running.remove(r)
+        if r in self.waiting:
+            self.waiting.remove(r)
+        if r.slot >= 0:
+            self.cache.release(r.slot)
+            r.slot = -1
+        r.cached_len = 0
+        r.keep_session = False
+        r.status = RequestStatus.FINISHED
+
+    def _evict_parked(self) -> bool:
+        """Take the cache of the session parked longest; False if none is parked."""
+        if not self.parked:
+            return False
+        r = self.parked.pop(0)
+        self.cache.release(r.slot)
+        r.slot = -1
+        r.cached_len = 0
+        self.num_evictions += 1
+        return True
 
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
@@ -113,6 +177,8 @@ class Scheduler:
 
         preempted = False
         while plan and not self.cache.can_extend([(p.request.slot, p.start + p.num_tokens) for p in plan]):
+            if self._evict_parked():
+                continue
             if len(self.running) == 1:
                 raise OutOfPages("the only running request does not fit into the cache")
             victim = max(self.running, key=lambda r: r.admitted_at)
@@ -121,13 +187,17 @@ class Scheduler:
             budget += sum(p.num_tokens for p in plan if p.request is victim)
             plan = [p for p in plan if p.request is not victim]
 
-        while not preempted and budget > 0 and self.cache.num_free_slots > 0:
+        while not preempted and budget > 0:
             r = next((w for w in self.waiting if chosen is None or w.request_id in chosen), None)
             if r is None:
+                break
+            if self.cache.num_free_slots == 0 and not self._evict_parked():
                 break
             n = min(r.extend_len, self.prefill_chunk, budget)
             slot = self.cache.admit()
             wants = [(p.request.slot, p.start + p.num_tokens) for p in plan] + [(slot, n)]
+            while not self.cache.can_extend(wants) and self._evict_parked():
+                pass
             if not self.cache.can_extend(wants):
                 self.cache.release(slot)
                 if not self.running:
@@ -165,8 +235,11 @@ class Scheduler:
             if p.samples:
                 r.append_token(next(it))
                 if r.finished:
-                    self.cache.release(r.slot)
-                    r.slot = -1
                     self.running.remove(r)
+                    if r.keep_session:
+                        self.parked.append(r)
+                    else:
+                        self.cache.release(r.slot)
+                        r.slot = -1
                     done.append(r)
         return done

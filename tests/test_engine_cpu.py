@@ -45,3 +45,43 @@ def test_cuts_match_plain(tmp_path, which):
         err = (got.double() - want).abs().max().item()
         assert err < 2e-5, (cuts, err)
     assert all(g.pool.num_held == 0 for g in runner.cache.groups)
+
+
+def test_page_size_and_batch_order_do_not_matter(tmp_path):
+    """The same three requests, stepped together in portions, with pages of 1, 4 and 16
+    tokens and with the entries of every step in both orders: the same logits."""
+    d = make_model_dir(tmp_path, "B")
+    cfg, w = plain.read_model_dir(d)
+    reqs = [random_tokens(n, cfg["vocab_size"], 60 + i) for i, n in enumerate((19, 7, 12))]
+    want = [plain.model_logits_fast(t, w, cfg) for t in reqs]
+
+    def run(page_size, reverse):
+        runner = make_runner(d, page_size, 64 // page_size + 4)
+        slots = [runner.admit() for _ in reqs]
+        got = [[] for _ in reqs]
+        at = [0] * len(reqs)
+        for portion in (5, 1, 6, 1, 8):
+            entries, who = [], []
+            for i, t in enumerate(reqs):
+                part = t[at[i] : at[i] + portion]
+                if part:
+                    entries.append(StepEntry(slots[i], part, list(range(len(part)))))
+                    who.append(i)
+                    at[i] += len(part)
+            if reverse:
+                entries, who = entries[::-1], who[::-1]
+            rows = runner.step(entries)
+            start = 0
+            for e, i in zip(entries, who):
+                got[i].append(rows[start : start + len(e.tokens)])
+                start += len(e.tokens)
+        for s in slots:
+            runner.release(s)
+        return [torch.cat(g) for g in got]
+
+    base = run(4, False)
+    for g, x in zip(base, want):
+        assert (g.double() - x).abs().max().item() < 2e-5
+    for page_size, reverse in ((1, False), (16, False), (4, True), (16, True)):
+        for g, b in zip(run(page_size, reverse), base):
+            assert (g - b).abs().max().item() < 1e-5, (page_size, reverse)

@@ -42,6 +42,66 @@ def test_chunked_prefill_and_preemption_do_not_change_tokens(tmp_path):
     assert all(g.pool.num_held == 0 for g in small.cache.groups)
 
 
+def test_session_continues_from_its_cache_and_is_released(tmp_path):
+    """Two turns as in tests/test_paged_generate_engine.cpp:555-663: the second turn keeps the
+    history, counts its own new tokens only, runs only the new tokens, and generates what a
+    fresh request over the whole history generates."""
+    d = make_model_dir(tmp_path, "B")
+    cfg, w = plain.read_model_dir(d)
+    first, second = random_tokens(11, 503, 31), random_tokens(5, 503, 32)
+    gen1 = plain.generate_greedy(first, w, cfg, 4)
+    gen2 = plain.generate_greedy(first + gen1 + second, w, cfg, 3)
+    eng = cpu_engine(d, page_size=8, num_pages=8, max_requests=2, prefill_chunk=4)
+    r = eng.add_request(first, 4, keep_session=True)
+    eng.run_until_finished()
+    assert r.finished and r.generated == gen1 and r.slot >= 0
+    held = eng.cache.groups[0].pool.num_held
+    assert held > 0 and r.cached_len == len(first) + 3  # the last token drawn is not cached yet
+    eng.append_input_tokens(r, second, 3)
+    assert not r.finished and r.generated == [] and r.prompt_len == len(first) + 4 + len(second)
+    assert r.cached_len == len(first) + 3 and r.extend_len == len(second) + 1
+    steps_before = eng.num_steps
+    eng.run_until_finished()
+    assert r.finished and r.generated == gen2 and r.tokens == first + gen1 + second + gen2
+    # 6 tokens in portions of 4 (two steps, the second draws), then two decode steps
+    assert eng.num_steps - steps_before == 4
+    eng.release_request(r)
+    assert r.slot == -1 and all(g.pool.num_held == 0 for g in eng.cache.groups)
+    # a request that was not kept is recomputed whole when it is continued
+    r2 = eng.add_request(first, 4)
+    eng.run_until_finished()
+    assert r2.slot == -1 and r2.generated == gen1
+    eng.append_input_tokens(r2, second, 3)
+    assert r2.cached_len == 0
+    eng.run_until_finished()
+    assert r2.generated == gen2 and all(g.pool.num_held == 0 for g in eng.cache.groups)
+
+
+def test_parked_sessions_lose_their_cache_before_running_requests_are_preempted(tmp_path):
+    d = make_model_dir(tmp_path, "A")
+    cfg, w = plain.read_model_dir(d)
+    a, b, c = (random_tokens(n, 256, 40 + i) for i, n in enumerate((9, 10, 14)))
+    eng = cpu_engine(d, page_size=4, num_pages=8, max_requests=3)
+    ra = eng.add_request(a, 3, keep_session=True)
+    eng.run_until_finished()
+    rb = eng.add_request(b, 3, keep_session=True)
+    eng.run_until_finished()
+    assert eng.scheduler.parked == [ra, rb] and eng.cache.groups[0].pool.num_free == 2
+    rc = eng.add_request(c, 4)  # needs 5 pages at its longest: the session parked longest goes first
+    eng.run_until_finished()
+    assert rc.generated == plain.generate_greedy(c, w, cfg, 4)
+    assert eng.scheduler.num_evictions == 1 and eng.scheduler.num_preemptions == 0
+    assert ra.slot == -1 and ra.cached_len == 0 and rb.slot >= 0 and eng.scheduler.parked == [rb]
+    # the evicted session can still go on: from its first token
+    more = random_tokens(2, 256, 50)
+    eng.append_input_tokens(ra, more, 2)
+    eng.run_until_finished()
+    assert ra.generated == plain.generate_greedy(a + plain.generate_greedy(a, w, cfg, 3) + more, w, cfg, 2)
+    eng.release_request(ra)
+    eng.release_request(rb)
+    assert all(g.pool.num_held == 0 for g in eng.cache.groups)
+
+
 def test_eos_is_appended_and_ends_the_request(tmp_path):
     d = make_model_dir(tmp_path, "A")
     cfg, w = plain.read_model_dir(d)
