@@ -164,18 +164,21 @@ struct RowState {
     float m[RT], l[RT];            // running maximum (base 2) and this lane's share of the sum
 };
 
-template <int DK, int RT>
+// LOAD_Q = false: the caller has filled st.qv itself
+template <int DK, int RT, bool LOAD_Q = true>
 __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT]) {
     const int c = (threadIdx.x % LLE_WAVE) / 16;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
+        if (LOAD_Q) {
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) {
-            if (row[t].q) {
-                st.qv[t][ks] = *(const bf16x8*)(row[t].q + 32 * ks + 8 * c);
-            } else {
+            for (int ks = 0; ks < DK; ++ks) {
+                if (row[t].q) {
+                    st.qv[t][ks] = *(const bf16x8*)(row[t].q + 32 * ks + 8 * c);
+                } else {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) st.qv[t][ks][i] = (bf16_t)0.0f;
+                    for (int i = 0; i < 8; ++i) st.qv[t][ks][i] = (bf16_t)0.0f;
+                }
             }
         }
 #pragma unroll
@@ -316,7 +319,7 @@ struct StepOperands {
 // meet again): the loop runs an even number of steps, loads past the end go to a page that is
 // there, and the CALLER has limited the rows' `pos` to the last key of step_end - 1, so that a
 // step past the end is masked out whole.
-template <int DK, int RT>
+template <int DK, int RT, bool LOAD_Q = true>
 __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT],
                                             const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ table,
                                             int kvh, int nkv, int P, int64_t page_stride, int step_begin,
@@ -324,7 +327,7 @@ __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo 
     constexpr int D = DK * 32;
     const int lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    init_rows<DK, RT>(st, row);
+    init_rows<DK, RT, LOAD_Q>(st, row);
     const int64_t k_lane = (int64_t)kvh * P * D + (int64_t)r16 * D + 8 * c;
     const int64_t v_lane = ((int64_t)nkv + kvh) * P * D + (int64_t)r16 * P + 4 * c;
     // Page and offset of a step's first key are carried from step to step instead of divided
@@ -399,18 +402,153 @@ __device__ __forceinline__ RowInfo make_row(const bf16_t* q, int r, int nrows, i
     return info;
 }
 
+// What the decode kernel needs to do the step before it as well: the RMSNorm of each q and k
+// head, the rotation over the whole head, and the write of the new K and V into the pages.
+// (Decode steps are short and every launch has a price; the prompt path keeps its own kernel.)
+struct FusedQKV {
+    const bf16_t* qkv;      // [N, (nq + 2 nkv) * D] as the projection left it
+    const int32_t* slots;   // [N] place of each token in the pages (page * P + offset), < 0: not written
+    const void* q_weight;   // [D] or nullptr: no norm
+    const void* k_weight;
+    int weight_dtype;
+    const float* cos_sin;   // [N, D / 2, 2]
+    float eps;
+    int write_kv;
+};
+
+__device__ __forceinline__ void load_weights8(const void* w, int e, int dtype, float (&out)[8]) {
+    if (dtype == LLE_F32) {
+        const float4 a = *(const float4*)((const float*)w + e), b = *(const float4*)((const float*)w + e + 4);
+        out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+    } else {
+        const bf16x8 v = *(const bf16x8*)((const bf16_t*)w + e);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
+    }
+}
+
+// Q^T operands of the lane's row from the raw projection: norm over the head (its 4 * DK * 8
+// elements sit in the four lanes r16 + 16 c), weight, rotation.  Element 32 ks + 8 c + i and its
+// partner D / 2 further on are both in this lane (DK is even).  Rounded to bfloat16 as the
+// separate kernel rounds q.
+template <int DK>
+__device__ __forceinline__ void fused_q_row(bf16x8 (&qv)[DK], const bf16_t* src, const FusedQKV& f, int64_t tok) {
+    static_assert(DK % 2 == 0, "rotation partners lie in one lane only for an even number of 32-element blocks");
+    constexpr int D = DK * 32;
+    const int c = (threadIdx.x % LLE_WAVE) / 16;
+    float x[DK][8];
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) {
+        bf16x8 v;
+        if (src) {
+            v = *(const bf16x8*)(src + 32 * ks + 8 * c);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = (bf16_t)0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[ks][i] = (float)v[i];
+    }
+    if (f.q_weight) {
+        float ss = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += x[ks][i] * x[ks][i];
+        ss += __shfl_xor(ss, 16, LLE_WAVE);
+        ss += __shfl_xor(ss, 32, LLE_WAVE);
+        const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) {
+            float w[8];
+            load_weights8(f.q_weight, 32 * ks + 8 * c, f.weight_dtype, w);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[ks][i] = x[ks][i] * inv * w[i];
+        }
+    }
+    if (src) {
+#pragma unroll
+        for (int ks = 0; ks < DK / 2; ++ks) {
+            const float4* tab = (const float4*)(f.cos_sin + (tok * (D / 2) + 32 * ks + 8 * c) * 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 t = tab[i];  // cos, sin of element 2 i, then of 2 i + 1
+                const float a0 = x[ks][2 * i], b0 = x[ks + DK / 2][2 * i];
+                const float a1 = x[ks][2 * i + 1], b1 = x[ks + DK / 2][2 * i + 1];
+                x[ks][2 * i] = a0 * t.x - b0 * t.y;
+                x[ks + DK / 2][2 * i] = b0 * t.x + a0 * t.y;
+                x[ks][2 * i + 1] = a1 * t.z - b1 * t.w;
+                x[ks + DK / 2][2 * i + 1] = b1 * t.z + a1 * t.w;
+            }
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) qv[ks][i] = (bf16_t)x[ks][i];
+}
+
+// One wavefront: K (norm, weight, rotation) and V of token `tok`, kv head `kvh`, into the pages.
+// Lane l takes elements l, l + 64, ... < D / 2 and their partners D / 2 further on.
+template <int DK>
+__device__ __forceinline__ void fused_kv_write(const FusedQKV& f, int64_t tok, int kvh, int nq, int nkv,
+                                               bf16_t* kv_layer, int P, int64_t page_stride) {
+    constexpr int D = DK * 32, HALF = D / 2, PER = (HALF + LLE_WAVE - 1) / LLE_WAVE;
+    const int lane = threadIdx.x % LLE_WAVE;
+    const int slot = f.slots[tok];
+    if (slot < 0) return;
+    const int page = slot / P, off = slot - page * P;
+    const bf16_t* ksrc = f.qkv + (tok * (nq + 2 * nkv) + nq + kvh) * D;
+    const bf16_t* vsrc = ksrc + (int64_t)nkv * D;
+    bf16_t* page_base = kv_layer + (int64_t)page * page_stride;
+    bf16_t* kdst = page_base + ((int64_t)kvh * P + off) * D;
+    bf16_t* vdst = page_base + ((int64_t)nkv + kvh) * P * D + off;  // element e at vdst[e * P]
+    float lo[PER], hi[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int e = lane + LLE_WAVE * j;
+        lo[j] = e < HALF ? (float)ksrc[e] : 0.f;
+        hi[j] = e < HALF ? (float)ksrc[e + HALF] : 0.f;
+        ss += lo[j] * lo[j] + hi[j] * hi[j];
+    }
+    if (f.k_weight) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int e = lane + LLE_WAVE * j;
+            if (e < HALF) {
+                lo[j] = lo[j] * inv * load_as_f32(f.k_weight, e, f.weight_dtype);
+                hi[j] = hi[j] * inv * load_as_f32(f.k_weight, e + HALF, f.weight_dtype);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int e = lane + LLE_WAVE * j;
+        if (e < HALF) {
+            const float2 t = *(const float2*)(f.cos_sin + (tok * HALF + e) * 2);
+            kdst[e] = (bf16_t)(lo[j] * t.x - hi[j] * t.y);
+            kdst[e + HALF] = (bf16_t)(hi[j] * t.x + lo[j] * t.y);
+            vdst[(int64_t)e * P] = vsrc[e];
+            vdst[(int64_t)(e + HALF) * P] = vsrc[e + HALF];
+        }
+    }
+}
+
 // Requests whose rows (q_len * group) fit one 16-row tile: decoded tokens and very
 // short portions.  grid = (requests, kv heads, splits).
 #ifndef DEC_WAVES
 #define DEC_WAVES 4
 #endif
-template <int DK>
+template <int DK, bool FUSED>
 __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int ws_stride, int nq, int nkv, int P, int64_t page_stride, int max_pages,
-    int window, float scale_log2) {
+    int window, float scale_log2, FusedQKV fused) {
     constexpr int D = DK * 32;
     extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
     float* s_o = smem;
@@ -429,7 +567,8 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int c = lane / 16, r16 = lane % 16;
     const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
 
-    RowInfo row[1] = {make_row(q, r16, nrows, G, q_start, past, nq, kvh, D, window)};
+    // FUSED: q is made here from the projection; the row's pointer only says that the row exists
+    RowInfo row[1] = {make_row(FUSED ? fused.qkv : q, r16, nrows, G, q_start, past, nq, kvh, D, window)};
     const int lo_min = window > 0 ? max(0, past - window + 1) : 0;
     const int hi = kv_len - 1;
     const int first = lo_min / KSTEP, last = hi / KSTEP;
@@ -438,10 +577,32 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int se = min(last + 1, sb + per_split);
     // keys of later splits are not this workgroup's: attend_rows may run a step past `se`
     row[0].pos = min(row[0].pos, se * KSTEP - 1);
+    if (FUSED) {
+        // The new keys and values of this head that lie in this workgroup's share of the steps
+        // go into the pages first; no other workgroup reads them in this launch, and this one
+        // reads them only after the barrier, by which the stores are done.
+        if (fused.write_kv) {
+            for (int t = wave; t < q_len; t += DEC_WAVES) {
+                const int step_of = (past + t) / KSTEP;
+                if (step_of >= sb && step_of < se)
+                    fused_kv_write<DK>(fused, (int64_t)q_start + t, kvh, nq, nkv, kv_layer, P, page_stride);
+            }
+        }
+        __syncthreads();
+    }
 
     RowState<DK, 1> st;
-    attend_rows<DK, 1>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi,
-                       scale_log2);
+    if constexpr (FUSED) {
+        const bf16_t* src = nullptr;
+        int64_t tok = 0;
+        if (r16 < nrows) {
+            tok = (int64_t)q_start + r16 / G;
+            src = fused.qkv + (tok * (nq + 2 * nkv) + kvh * G + r16 % G) * D;
+        }
+        fused_q_row<DK>(st.qv[0], src, fused, tok);
+    }
+    attend_rows<DK, 1, !FUSED>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min,
+                               hi, scale_log2);
 
     // merge the wavefronts (rows that do not exist are not worth the LDS traffic)
     if (r16 < nrows) {
@@ -728,28 +889,52 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     }
 }
 
+template <int DK, bool FUSED>
+static int launch_decode(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_tables, const int32_t* seq_slots,
+                         const int32_t* cu_tokens, const int32_t* kv_lens, bf16_t* out, float* ws_o, float* ws_ml,
+                         int ws_stride, int S, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
+                         float scale_log2, int nsplit, const FusedQKV& fused, hipStream_t stream) {
+    constexpr int D = DK * 32;
+    const size_t smem = (size_t)(DEC_WAVES * 16 * D + 2 * DEC_WAVES * 16) * sizeof(float);
+    if (smem > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)mfma_decode_kernel<DK, FUSED>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (e != hipSuccess) return (int)e;
+    }
+    mfma_decode_kernel<DK, FUSED><<<dim3(S, nkv, nsplit), DEC_WAVES * LLE_WAVE, smem, stream>>>(
+        q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nq, nkv, P,
+        page_stride, max_pages, window, scale_log2, fused);
+    return 0;
+}
+
 template <int DK>
-static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* block_tables,
+static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_tables,
                        const int32_t* seq_slots, const int32_t* cu_tokens, const int32_t* kv_lens,
                        const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
                        int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
                        int run_decode, int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                       hipStream_t stream) {
+                       const FusedQKV& fused, hipStream_t stream) {
     constexpr int D = DK * 32;
     const int G = nq / nkv;
     if (!run_decode) nsplit_decode = 1;
     if (!run_prefill) nsplit_prefill = 1;
     const int ws_stride = nsplit_decode > nsplit_prefill ? nsplit_decode : nsplit_prefill;
+    if (fused.qkv && (run_prefill || !run_decode || DK % 2 != 0)) return (int)hipErrorInvalidValue;
     if (run_decode) {
-        const size_t smem = (size_t)(DEC_WAVES * 16 * D + 2 * DEC_WAVES * 16) * sizeof(float);
-        if (smem > 64 * 1024) {
-            hipError_t e = hipFuncSetAttribute((const void*)mfma_decode_kernel<DK>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-            if (e != hipSuccess) return (int)e;
+        int e;
+        if constexpr (DK % 2 == 0) {
+            e = fused.qkv ? launch_decode<DK, true>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o,
+                                                    ws_ml, ws_stride, S, nq, nkv, P, page_stride, max_pages, window,
+                                                    scale_log2, nsplit_decode, fused, stream)
+                          : launch_decode<DK, false>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out,
+                                                     ws_o, ws_ml, ws_stride, S, nq, nkv, P, page_stride, max_pages,
+                                                     window, scale_log2, nsplit_decode, fused, stream);
+        } else {
+            e = launch_decode<DK, false>(q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml,
+                                         ws_stride, S, nq, nkv, P, page_stride, max_pages, window, scale_log2,
+                                         nsplit_decode, fused, stream);
         }
-        mfma_decode_kernel<DK><<<dim3(S, nkv, nsplit_decode), DEC_WAVES * LLE_WAVE, smem, stream>>>(
-            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nq, nkv, P,
-            page_stride, max_pages, window, scale_log2);
+        if (e != 0) return e;
     }
     if (run_prefill) {
         constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT_OF(DK);
@@ -771,12 +956,12 @@ static int launch_mfma(const bf16_t* q, const bf16_t* kv_layer, const int32_t* b
 // with q_len * group <= 16 rows are the decode kernel's); with ns = max(nsplit_decode,
 // nsplit_prefill) > 1 the workspaces ws_o [N * nq * ns * d] and ws_ml [N * nq * ns * 2]
 // floats are needed (ns <= 64).
-extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, const void* block_tables,
-                                        const void* seq_slots, const void* cu_tokens, const void* kv_lens,
-                                        const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
-                                        int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
-                                        int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
-                                        int nsplit_prefill, int max_q_len, hipStream_t stream) {
+static int paged_attention_mfma(const void* q, void* kv_layer, const void* block_tables, const void* seq_slots,
+                                const void* cu_tokens, const void* kv_lens, const void* token_seq, void* out,
+                                void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d, int page_size,
+                                int64_t page_stride, int max_pages, int window, float scale, int run_decode,
+                                int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
+                                const FusedQKV& fused, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv > 65535) return (int)hipErrorInvalidValue;
@@ -785,11 +970,11 @@ extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, con
     const float scale_log2 = scale * 1.44269504088896340736f;
 #define LLE_ATT_CASE(DKV)                                                                                          \
     case DKV:                                                                                                      \
-        return launch_mfma<DKV>((const bf16_t*)q, (const bf16_t*)kv_layer, (const int32_t*)block_tables,            \
+        return launch_mfma<DKV>((const bf16_t*)q, (bf16_t*)kv_layer, (const int32_t*)block_tables,                  \
                                 (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
                                 (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
                                 page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit_decode,   \
-                                run_prefill, nsplit_prefill, max_q_len, stream);
+                                run_prefill, nsplit_prefill, max_q_len, fused, stream);
     switch (d / 32) {
         LLE_ATT_CASE(1)
         LLE_ATT_CASE(2)
@@ -802,4 +987,45 @@ extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, con
     }
 #undef LLE_ATT_CASE
     return (int)hipErrorInvalidValue;
+}
+
+extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, const void* block_tables,
+                                        const void* seq_slots, const void* cu_tokens, const void* kv_lens,
+                                        const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
+                                        int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
+                                        int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
+                                        int nsplit_prefill, int max_q_len, hipStream_t stream) {
+    const FusedQKV none = {};
+    return paged_attention_mfma(q, (void*)kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
+                                ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, run_decode,
+                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, none, stream);
+}
+
+// Decode steps only (every request has at most 16 / group tokens), head_dim a multiple of 64, a
+// rotation over the whole head: the q/k norm, the rotation and the write of the new K and V
+// (write_kv != 0; slots [N], < 0: not written) happen inside the attention launch.  qkv is
+// [N, (nq + 2 nkv) * d] as the projection left it; q_weight / k_weight [d] or null; cos_sin
+// [N, d / 2, 2] float32.
+extern "C" int lle_qk_norm_rope_attention_decode(const void* qkv, const void* slots, const void* q_weight,
+                                                 const void* k_weight, int weight_dtype, const void* cos_sin,
+                                                 float eps, int write_kv, void* kv_layer, const void* block_tables,
+                                                 const void* seq_slots, const void* cu_tokens, const void* kv_lens,
+                                                 const void* token_seq, void* out, void* ws_o, void* ws_ml, int N,
+                                                 int S, int nq, int nkv, int d, int page_size, int64_t page_stride,
+                                                 int max_pages, int window, float scale, int nsplit_decode,
+                                                 hipStream_t stream) {
+    if (!qkv || !cos_sin || !slots || d % 64 != 0) return (int)hipErrorInvalidValue;
+    if ((q_weight == nullptr) != (k_weight == nullptr)) return (int)hipErrorInvalidValue;
+    FusedQKV fused;
+    fused.qkv = (const bf16_t*)qkv;
+    fused.slots = (const int32_t*)slots;
+    fused.q_weight = q_weight;
+    fused.k_weight = k_weight;
+    fused.weight_dtype = weight_dtype;
+    fused.cos_sin = (const float*)cos_sin;
+    fused.eps = eps;
+    fused.write_kv = write_kv;
+    return paged_attention_mfma(nullptr, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
+                                ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, 1,
+                                nsplit_decode, 0, 1, 1, fused, stream);
 }

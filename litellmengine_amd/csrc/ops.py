@@ -299,7 +299,62 @@ class HipOps:
                   int(run_prefill), ns_prefill, max_q_len)
         return out
 
+    def can_fuse_rope_attention(self, dtype, head_dim: int, rotary_dim: int, page_size: int, group: int,
+                                max_q_len: int, max_kv_len: int, num_seqs: int) -> bool:
+        """Whether qk_norm_rope_attention takes this step: bfloat16, a rotation over the whole head
+        of a multiple of 64 elements, and only requests of at most 16 / group tokens (decode steps)."""
+        return (dtype == torch.bfloat16 and head_dim % 64 == 0 and head_dim <= self.MAX_HEAD_DIM
+                and rotary_dim == head_dim and page_size % 16 == 0 and 0 < max_q_len and max_q_len * group <= 16
+                and max_kv_len > 0 and num_seqs <= 65535 and not self.force_generic_attention
+                and not self.force_separate_rope)
+
+    def qk_norm_rope_attention(self, qkv, slots, q_weight, k_weight, cos_sin, eps: float, kv_layer, nq: int,
+                               nkv: int, d: int, write_kv: bool, block_table, seq_slots, cu_tokens, kv_lens,
+                               token_seq, window: Optional[int], scale: float, max_kv_len: int) -> torch.Tensor:
+        """qk_norm_rope_write and paged_attention of a decode step in one launch (see
+        can_fuse_rope_attention): the workgroup whose keys include a new token's position writes
+        its K and V, every workgroup norms and rotates the q rows it multiplies."""
+        _dev(qkv, "qkv", torch.bfloat16)
+        _dev(kv_layer, "kv_layer", torch.bfloat16)
+        _dev(cos_sin, "cos_sin", torch.float32)
+        for t, name in ((slots, "slots"), (block_table, "block_table"), (seq_slots, "seq_slots"),
+                        (cu_tokens, "cu_tokens"), (kv_lens, "kv_lens"), (token_seq, "token_seq")):
+            _dev(t, name, torch.int32)
+        N = qkv.shape[0]
+        page_size = kv_layer.shape[3]
+        _need(qkv.shape[1] == (nq + 2 * nkv) * d, "qkv must be [N, (nq + 2 nkv) * d]")
+        _need(tuple(kv_layer.shape[1:]) == (2, nkv, page_size, d), "kv_layer must be [pages, 2, nkv, page_size, d]")
+        _need(slots.shape == (N,) and token_seq.shape == (N,), "slots and token_seq must be [N]")
+        _need(cos_sin.shape == (N, d // 2, 2), f"cos_sin must be [{N}, {d // 2}, 2]")
+        _need((q_weight is None) == (k_weight is None), "q and k norm weights come together")
+        wcode = 0
+        if q_weight is not None:
+            _dev(q_weight, "q_weight")
+            _dev(k_weight, "k_weight", q_weight.dtype)
+            _need(q_weight.shape == (d,) and k_weight.shape == (d,), f"q/k norm weights must be [{d}]")
+            wcode = dtype_code(q_weight.dtype)
+        S = seq_slots.shape[0]
+        _need(cu_tokens.shape == (S + 1,) and kv_lens.shape == (S,), "cu_tokens [S + 1], kv_lens [S]")
+        _need(nq % nkv == 0 and d % 64 == 0 and page_size % 16 == 0 and S <= 65535,
+              "the fused decode attention does not take these sizes")
+        win = int(window) if window else 0
+        ns = self.decode_splits(S, nkv, max_kv_len, win)
+        out = torch.empty((N, nq * d), dtype=torch.bfloat16, device=qkv.device)
+        ws_o = ws_ml = None
+        if ns > 1:
+            ws_o = torch.empty((N * nq * ns * d,), dtype=torch.float32, device=qkv.device)
+            ws_ml = torch.empty((N * nq * ns * 2,), dtype=torch.float32, device=qkv.device)
+        self._run("attention", "lle_qk_norm_rope_attention_decode",
+                  [_P, _P, _P, _P, _I, _P, _F, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I,
+                   _F, _I, _P],
+                  _ptr(qkv), _ptr(slots), _ptr(q_weight), _ptr(k_weight), wcode, _ptr(cos_sin), float(eps),
+                  int(bool(write_kv)), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens),
+                  _ptr(kv_lens), _ptr(token_seq), _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size,
+                  kv_layer.stride(0), block_table.shape[1], win, float(scale), ns)
+        return out
+
     force_generic_attention = False  # tests flip this to compare the two families of kernels
+    force_separate_rope = False      # tests flip this to compare the fused decode step with its two halves
     # measured on MI355X: about one workgroup per CU and at least 16 32-key steps (four per
     # wavefront) per split are best; more splits cost more in partial results than they gain
     DECODE_TARGET_BLOCKS = 256

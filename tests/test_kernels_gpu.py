@@ -323,6 +323,58 @@ def test_matrix_core_attention(nq, nkv, d, P, window, lens):
     assert (got.double() - generic.double()).abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32, None])
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(32, 8, 128, 16, None), (4, 4, 64, 32, None), (16, 2, 64, 16, 50),
+                                               (6, 1, 192, 48, None), (8, 2, 256, 16, 900)])
+@pytest.mark.parametrize("lens", [
+    [(1999, 1), (640, 1), (31, 1), (0, 1)],   # long contexts: the new key lies in the last of several key splits
+    [(15, 1), (16, 1), (47, 1)],              # the new key is the last of a page / the first of a new one
+    [(100, 2), (31, 2), (0, 1), (2047, 2)],   # two tokens of a request in one step, across a page's and a step's edge
+])
+def test_fused_decode_attention_equals_its_two_halves(wdtype, nq, nkv, d, P, window, lens):
+    """Norm, rotation, cache write and attention of a decode step in one launch against the
+    two kernels it replaces, on the same inputs: the same pages afterwards, the same output."""
+    group = nq // nkv
+    lens = [(p, min(l, 16 // group)) for p, l in lens if 16 // group >= 1]
+    need = max((p + l + P - 1) // P for p, l in lens)
+    args, mq, mk = attention_case(torch.bfloat16, nq, nkv, d, P, window, lens,
+                                  pages=sum((p + l + P - 1) // P for p, l in lens) + 3, max_pages=need + 1)
+    _, kv, table, seq_slots, cu, kv_lens, token_seq, _, scale = args
+    N = int(cu[-1])
+    qkv = rnd((N, (nq + 2 * nkv) * d), torch.bfloat16, 70, 1.5)
+    positions, slots = [], []
+    for s, (past, ql) in enumerate(lens):
+        for t in range(ql):
+            pos = past + t
+            positions.append(pos)
+            slots.append(int(table[int(seq_slots[s]), pos // P]) * P + pos % P)
+    positions = torch.tensor(positions, dtype=torch.int32).cuda()
+    slots = torch.tensor(slots, dtype=torch.int32).cuda()
+    i = torch.arange(d // 2, dtype=torch.float64)
+    inv = (1e6 ** (-(2.0 * i) / d)).float().cuda()
+    o = ops()
+    cs = o.rope_table(positions, inv)
+    qw = kw = None
+    if wdtype is not None:
+        qw = (1 + 0.2 * rnd((d,), torch.float32, 71)).to(wdtype)
+        kw = (1 + 0.2 * rnd((d,), torch.float32, 72)).to(wdtype)
+    assert o.can_fuse_rope_attention(torch.bfloat16, d, d, P, group, mq[1], mk, len(lens))
+    kv_a, kv_b = kv.clone(), kv.clone()
+    q = o.qk_norm_rope_write(qkv, slots, qw, kw, cs, d, 1e-5, kv_a, nq, nkv, d, True)
+    want = o.paged_attention(q, kv_a, table, seq_slots, cu, kv_lens, token_seq, window, scale, *mq, mk)
+    got = o.qk_norm_rope_attention(qkv, slots, qw, kw, cs, 1e-5, kv_b, nq, nkv, d, True, table, seq_slots, cu,
+                                   kv_lens, token_seq, window, scale, mk)
+    assert not torch.equal(kv_b, kv), "the new keys and values are written"
+    # both round the same 32-bit results to bfloat16; one unit in the last place where a product was fused differently
+    assert (kv_a.float() - kv_b.float()).abs().max() <= 2.0 ** -7 * kv_a.float().abs().max()
+    assert (got.double() - want.double()).abs().max() < 2e-2
+    # without writing (a layer that reads another layer's pages): the pages stay, q is still made
+    kv_c = kv_a.clone()
+    again = o.qk_norm_rope_attention(qkv, slots, qw, kw, cs, 1e-5, kv_c, nq, nkv, d, False, table, seq_slots, cu,
+                                     kv_lens, token_seq, window, scale, mk)
+    assert torch.equal(kv_c, kv_a) and (again.double() - want.double()).abs().max() < 2e-2
+
+
 def test_matrix_core_attention_far_key_and_window_edge():
     """A key hundreds of positions back is made to dominate, with the window
     ending exactly on it (seen) or one short of it (not seen)."""
