@@ -102,21 +102,23 @@ typedef float gf32x4 __attribute__((ext_vector_type(4)));
 //   RESID (the product before the norm): its result is the delta of the residual stream; the
 //     epilogue forms h = hidden + delta in 32-bit, writes it back, writes xw = h * w as the
 //     next product's input, and leaves the sum of h^2 over its 16 columns per row in
-//     ss_part[workgroup][16];
+//     ss_part[16][workgroups];
 //   SCALED (the product after the norm): adds up the parts, and multiplies its rows by r[m].
 struct NormFold {
     float* hidden;          // RESID: residual stream [M, N], read and written
     const void* weight;     // RESID: norm weight [N]
     int weight_dtype;
     bf16_t* xw;             // RESID: out, [M, N]
-    float* ss_out;          // RESID: out, [workgroups][16]
-    const float* ss_in;     // SCALED: [parts][16]
+    float* ss_out;          // RESID: out, [16][workgroups]
+    const float* ss_in;     // SCALED: [16][parts]
     int parts;              // SCALED
     float eps;              // SCALED
 };
 
 template <int MT, int NT, bool GATED, bool RESID, bool SCALED, typename TC, int SK_WAVES, int UNROLL>
-__global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
+// one tile of W and up to 16 rows of X: two workgroups of 16 wavefronts a CU (8 wavefronts a SIMD),
+// which 64 registers allow; the gated form measured faster with the registers it asks for
+__global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                          const bf16_t* __restrict__ W,
                                                                          TC* __restrict__ C, int M, int N, int K,
                                                                          NormFold fold) {
@@ -124,15 +126,19 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
     // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
     __shared__ float s_inv[16];
-    if (SCALED && threadIdx.x < 256) {  // r[m] from the parts, 16 threads a row
-        const int m = threadIdx.x / 16, j = threadIdx.x % 16;
-        float part = 0.f;
-        for (int b = j; b < fold.parts; b += 16) part += fold.ss_in[b * 16 + m];
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) part += __shfl_xor(part, o, LLE_WAVE);
-        if (j == 0) s_inv[m] = 1.0f / sqrtf(part / (float)K + fold.eps);
-    }
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    // SCALED: wavefront m adds up the parts of row m.  The first parts are asked for now and
+    // added after the products, so that their way from memory is not waited for up front.
+    static_assert(!SCALED || SK_WAVES == 16, "one wavefront per row of the norm");
+    constexpr int EARLY_PARTS = GATED ? 0 : 4;  // the gated form has no registers to spare for them
+    float early[EARLY_PARTS + 1];
+    if (SCALED) {
+#pragma unroll
+        for (int i = 0; i < EARLY_PARTS; ++i) {
+            const int b = lane + LLE_WAVE * i;
+            early[i] = b < fold.parts ? fold.ss_in[(int64_t)wave * fold.parts + b] : 0.f;
+        }
+    }
     const int c = lane / 16, r16 = lane % 16;
     const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
     // RESID: thread (m, n) of the first 256 owns element [m][n0 + n]; what it needs of the
@@ -217,6 +223,15 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
             }
         }
     }
+    if (SCALED) {
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < EARLY_PARTS; ++i) part += early[i];
+        for (int b = lane + LLE_WAVE * EARLY_PARTS; b < fold.parts; b += LLE_WAVE)
+            part += fold.ss_in[(int64_t)wave * fold.parts + b];
+        part = wave_sum(part);
+        if (lane == 0) s_inv[wave] = 1.0f / sqrtf(part / (float)K + fold.eps);
+    }
     // lane holds C^T[n = 4c + i][m = r16]
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_kernel(const b
             }
 #pragma unroll
             for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, LLE_WAVE);
-            if (n == 0) fold.ss_out[(int64_t)blockIdx.x * 16 + m] = sq;
+            if (n == 0) fold.ss_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
         }
         return;
     }
@@ -319,7 +334,7 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
 
 // The product BEFORE a folded norm: delta = X W^T [M, N] is added into `hidden` (float32 [M, N],
 // in place), xw = hidden * norm_weight goes to `xw` (bfloat16 [M, N]) and the sums of squares of
-// the new hidden over each workgroup's 16 columns to ss_part [(N + 15) / 16][16].  1 <= M <= 16.
+// the new hidden over each workgroup's 16 columns to ss_part [16][(N + 15) / 16].  1 <= M <= 16.
 extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hidden, const void* norm_weight,
                                           int weight_dtype, void* xw, void* ss_part, int M, int N, int K,
                                           hipStream_t stream) {
@@ -337,7 +352,7 @@ extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hi
 }
 
 // The product AFTER a folded norm: X is the xw of lle_gemm_skinny_resid_bf16 and ss_part its
-// `parts` x 16 sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).  gated != 0:
+// 16 x `parts` sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).  gated != 0:
 // W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.  1 <= M <= 16.
 extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C, const void* ss_part, int parts,
                                            float eps, int M, int N, int K, int gated, hipStream_t stream) {

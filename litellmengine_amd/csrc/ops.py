@@ -144,8 +144,8 @@ class HipOps:
         _need(pre is None or fold is None, "a product takes a Prenormed or makes one, not both")
         if pre is not None:
             _dev(pre.sums, "sums", torch.float32)
-            parts = pre.sums.shape[0]
-            _need(pre.sums.shape == (parts, 16) and pre.xw.shape[1] == K, "sums of squares do not fit")
+            parts = pre.sums.shape[1]
+            _need(pre.sums.shape == (16, parts) and pre.xw.shape[1] == K, "sums of squares do not fit")
             _need(not gated or N % 2 == 0, "a gated weight has an even number of rows")
             out = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=xin.device)
             self._run("gemm", "lle_gemm_skinny_scaled_bf16", [_P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
@@ -157,7 +157,7 @@ class HipOps:
               f"residual stream {list(fold.hidden.shape)} does not fit a product [{M}, {N}]")
         _need(self.can_fold_norm(M, N, xin.dtype), f"a norm over {N} cannot be folded")
         xw = torch.empty((M, N), dtype=torch.bfloat16, device=xin.device)
-        sums = torch.empty(((N + 15) // 16, 16), dtype=torch.float32, device=xin.device)
+        sums = torch.empty((16, (N + 15) // 16), dtype=torch.float32, device=xin.device)
         self._run("gemm", "lle_gemm_skinny_resid_bf16", [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
                   _ptr(xin), _ptr(weight), _ptr(fold.hidden), _ptr(fold.weight), dtype_code(fold.weight.dtype),
                   _ptr(xw), _ptr(sums), M, N, K)

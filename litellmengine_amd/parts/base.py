@@ -70,12 +70,12 @@ class NormFold:
 @dataclasses.dataclass
 class Prenormed:
     """Normed rows whose last factor is still outstanding: row m of the norm's result is
-    `xw[m] * rsqrt(sum(sums[:, m]) / width + eps)`.  That factor commutes with a
+    `xw[m] * rsqrt(sum(sums[m]) / width + eps)`.  That factor commutes with a
     product, so the product that follows applies it to its own result.  Only
     `ops.linear` and `ops.gate_up_silu` take one, and each value is used once."""
 
     xw: torch.Tensor  # [N, width], hidden * norm weight, activation type
-    sums: torch.Tensor  # float32 [parts, 16]: sums of squares of hidden over column ranges, by row
+    sums: torch.Tensor  # float32 [16, parts]: row m's sums of squares of hidden over column ranges
     eps: float
 
 

@@ -123,8 +123,8 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         pre = o.linear(a, w1, fold=NormFold(h, nw, eps))
         want_h = hidden.double() + a.double() @ w1.double().t()
         assert (h.double() - want_h).abs().max() < 1e-4 * max(1.0, want_h.abs().max().item())
-        assert pre.sums.shape == ((H + 15) // 16, 16)
-        ss = pre.sums.double().sum(0)[:M]
+        assert pre.sums.shape == (16, (H + 15) // 16)
+        ss = pre.sums.double().sum(1)[:M]
         assert torch.allclose(ss, (want_h ** 2).sum(1), rtol=1e-5)
         normed = want_h * torch.rsqrt((want_h ** 2).mean(1, keepdim=True) + eps) * nw.double()
         y = normed @ w2.double().t()
