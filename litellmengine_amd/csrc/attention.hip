@@ -138,7 +138,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define NEG_BIG (-1.0e30f)
 #define LAZY_MAX 8.0f  // a row's reference maximum may lag its true one by this much (base 2)
-#define KSTEP 32  // keys per step: two 16-key tiles, each inside one page
+#define KSTEP 32  // keys per step: two 16-key tiles; pages hold a multiple of 16 keys
+#define KEY_OF_ROW(r, x) (8 * ((r) / 4) + 4 * (x) + (r) % 4)
 
 // What one lane knows about the query row it serves (row = lane % 16 of a 16-row tile).
 struct RowInfo {
@@ -152,10 +153,14 @@ struct RowInfo {
 //   S^T = K Q^T   (A = K tile [16 keys x 32], B = Q^T [32 x 16 rows])
 //   O^T += V^T P^T (A = V^T tile [16 d x 32 keys], B = P^T [32 keys x 16 rows])
 // With v_mfma_f32_16x16x32_bf16 a lane (c = lane / 16, r = lane % 16) holds, of a
-// result tile, column r and rows 4c..4c+3: for S^T that is query row r and keys
-// 4c..4c+3 — exactly what the B operand of the second product wants, so P never
-// leaves registers, and the softmax state of row r sits in the lanes r + 16c.
-// The k slots of the second product are (tile A keys 4c..4c+3, tile B keys 4c..4c+3).
+// result tile, column r and rows 4c..4c+3: for S^T that is query row r and four keys
+// — exactly what the B operand of the second product wants, so P never leaves
+// registers, and the softmax state of row r sits in the lanes r + 16c.
+// Which key a row of a K tile stands for is free.  The two tiles of a step take the keys
+//   row r of tile x  <->  key 8 (r / 4) + 4 x + r % 4   of the step        (KEY_OF_ROW)
+// so that a lane's eight scores (rows 4c..4c+3 of both tiles) are the CONSECUTIVE keys
+// 8c..8c+7: the V^T operand of the second product is then one 16-byte piece per lane
+// (keys 8c..8c+7 of one value element), inside one page.
 template <int DK, int RT>
 struct RowState {
     bf16x8 qv[RT][DK];             // Q^T operands of the lane's row
@@ -203,9 +208,9 @@ __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&
         for (int ks = 0; ks < DK; ++ks) asm volatile("" : "+v"(st.qv[t][ks]));
 }
 
-// One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key r16 of
-// half-tile x, elements 32 ks + 8 c .. + 7.  load_v(n): value element 16 n + r16, keys 4c..4c+3
-// of half-tile 0 then of half-tile 1.  Each operand is fetched once and used by all row tiles.
+// One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key
+// KEY_OF_ROW(r16, x) of the step, elements 32 ks + 8 c .. + 7.  load_v(n): value element
+// 16 n + r16, keys 8c..8c+7 of the step.  Each operand is fetched once and used by all row tiles.
 template <int DK, int RT, typename LoadK, typename LoadV>
 __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&row)[RT], LoadK load_k,
                                           LoadV load_v, int j0, float scale_log2) {
@@ -243,7 +248,7 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
         if (!(j0 >= st.open_lo[t] && j0 + KSTEP - 1 <= st.open_hi[t])) {  // same for the whole wavefront
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int j = j0 + 16 * (i / 4) + 4 * c + (i % 4);
+                const int j = j0 + 8 * c + i;  // score i of the lane: tile i / 4, row 4 c + i % 4
                 if (j < row[t].lo || j > row[t].pos) x[t][i] = NEG_BIG;
             }
         }
@@ -309,7 +314,7 @@ __device__ __forceinline__ void finish_rows(RowState<DK, RT>& st) {
 template <int DK>
 struct StepOperands {
     bf16x8 k[2][DK];
-    bf16x4 v[2 * DK][2];
+    bf16x8 v[2 * DK];
 };
 
 // The steps step_begin, step_begin + step_stride, ... < step_end with the operands loaded by
@@ -328,8 +333,11 @@ __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo 
     const int lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
     init_rows<DK, RT, LOAD_Q>(st, row);
-    const int64_t k_lane = (int64_t)kvh * P * D + (int64_t)r16 * D + 8 * c;
-    const int64_t v_lane = ((int64_t)nkv + kvh) * P * D + (int64_t)r16 * P + 4 * c;
+    // the lane's keys of tile x lie in the 16-key half r16 / 8 of the step, its eight V keys in half c / 2
+    const int k_half = r16 / 8, v_half = c / 2;
+    const int64_t k_lane[2] = {(int64_t)kvh * P * D + (int64_t)(KEY_OF_ROW(r16, 0) % 16) * D + 8 * c,
+                               (int64_t)kvh * P * D + (int64_t)(KEY_OF_ROW(r16, 1) % 16) * D + 8 * c};
+    const int64_t v_lane = ((int64_t)nkv + kvh) * P * D + (int64_t)r16 * P + 8 * (c % 2);
     // Page and offset of a step's first key are carried from step to step instead of divided
     // out each time (the page size is no constant), and the table is read one load ahead.  A
     // half wholly outside [lo_min, hi] may lie in a page that is not there: the page index is
@@ -354,23 +362,22 @@ __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo 
         }
     };
     auto load = [&](StepOperands<DK>& op) {
+        const bf16_t* half0 = kv_layer + (int64_t)page_id[0] * page_stride;
+        const bf16_t* half1 = kv_layer + (int64_t)page_id[1] * page_stride;
+        const bf16_t* kpage = (k_half ? half1 : half0) + (int64_t)(k_half ? page_off[1] : page_off[0]) * D;
+        const bf16_t* vp = (v_half ? half1 : half0) + v_lane + (v_half ? page_off[1] : page_off[0]);
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            const bf16_t* page = kv_layer + (int64_t)page_id[x] * page_stride;
-            const bf16_t* kp = page + k_lane + (int64_t)page_off[x] * D;
-            const bf16_t* vp = page + v_lane + page_off[x];
+        for (int x = 0; x < 2; ++x)
 #pragma unroll
-            for (int ks = 0; ks < DK; ++ks) op.k[x][ks] = *(const bf16x8*)(kp + 32 * ks);
+            for (int ks = 0; ks < DK; ++ks) op.k[x][ks] = *(const bf16x8*)(kpage + k_lane[x] + 32 * ks);
 #pragma unroll
-            for (int n = 0; n < 2 * DK; ++n) op.v[n][x] = *(const bf16x4*)(vp + (int64_t)16 * n * P);
-        }
+        for (int n = 0; n < 2 * DK; ++n) op.v[n] = *(const bf16x8*)(vp + (int64_t)16 * n * P);
         lookup();
     };
     auto multiply = [&](const StepOperands<DK>& op, int step) {
         tile_step<DK, RT>(
-            st, row, [&](int x, int ks) { return op.k[x][ks]; },
-            [&](int n) { return __builtin_shufflevector(op.v[n][0], op.v[n][1], 0, 1, 2, 3, 4, 5, 6, 7); },
-            step * KSTEP, scale_log2);
+            st, row, [&](int x, int ks) { return op.k[x][ks]; }, [&](int n) { return op.v[n]; }, step * KSTEP,
+            scale_log2);
     };
     StepOperands<DK> even, odd;
     lookup();
@@ -683,7 +690,7 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 // once per workgroup (all 256 threads, the next tile while this one is multiplied) and every
 // wavefront reads its matrix-core operands from there: 128 rows share one pass over the keys.
 //   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
-//   LDS V^T tile: [D][32 keys + 4]
+//   LDS V^T tile: [D][32 keys + 8]
 // row tiles per wavefront: two while the accumulators fit the register file
 #ifndef PRE_WAVES
 #define PRE_WAVES 8
@@ -703,7 +710,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     constexpr int PRE_RT = PRE_RT_OF(DK);
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
     constexpr int KROW = D + 8;       // elements per key row in LDS
-    constexpr int VROW = KSTEP + 4;   // elements per value-element row in LDS
+    constexpr int VROW = KSTEP + 8;   // elements per value-element row in LDS: 16-byte pieces stay aligned
     constexpr int TILE = KSTEP * KROW + D * VROW;
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * TILE];
 
@@ -822,9 +829,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
             const int piece = threadIdx.x + PRE_WAVES * LLE_WAVE * i;
             if (EVERY_THREAD_COPIES || piece < PIECES) {
                 *(bf16x8*)(tile + k_lds[i]) = stage_k[set][i];
-                bf16_t* dst = tile + v_lds[i];  // 8-byte aligned
-                *(bf16x4*)dst = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 0, 1, 2, 3);
-                *(bf16x4*)(dst + 4) = __builtin_shufflevector(stage_v[set][i], stage_v[set][i], 4, 5, 6, 7);
+                *(bf16x8*)(tile + v_lds[i]) = stage_v[set][i];
             }
         }
     };
@@ -841,12 +846,9 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
             const bf16_t* kt = lds + buf * TILE;
             const bf16_t* vt = kt + KSTEP * KROW;
             tile_step<DK, PRE_RT>(
-                st, row, [&](int x, int ks) { return *(const bf16x8*)(kt + (16 * x + r16) * KROW + 32 * ks + 8 * c); },
-                [&](int n) {
-                    const bf16_t* p = vt + (16 * n + r16) * VROW + 4 * c;
-                    return __builtin_shufflevector(*(const bf16x4*)p, *(const bf16x4*)(p + 16), 0, 1, 2, 3, 4, 5, 6, 7);
-                },
-                step * KSTEP, scale_log2);
+                st, row,
+                [&](int x, int ks) { return *(const bf16x8*)(kt + KEY_OF_ROW(r16, x) * KROW + 32 * ks + 8 * c); },
+                [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * VROW + 8 * c); }, step * KSTEP, scale_log2);
         }
         stash(buf ^ 1, set_c);
         __syncthreads();
