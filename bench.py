@@ -3,6 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
+    python bench.py --workload reference-0p6b [--dtype float32]   # the reference's own benchmark shape
+    python bench.py --workload mixed-32b [--layers L]             # a prompt chunk beside 63 decoded tokens
+
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
 `context` tokens.  Seeded random weights (bfloat16), uniform random token ids.
@@ -24,6 +27,19 @@ SIZES = dict(
     num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936,
     rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
 )
+# Qwen3-0.6B layer sizes: the model of the reference's published table (readme.md:62-66)
+SIZES_0P6B = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=28, hidden_size=1024,
+    num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072, vocab_size=151936,
+    rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=True,
+)
+# Qwen3-32B layer sizes
+SIZES_32B = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", num_hidden_layers=64, hidden_size=5120,
+    num_attention_heads=64, num_key_value_heads=8, head_dim=128, intermediate_size=25600, vocab_size=151936,
+    rope_theta=1000000.0, rms_norm_eps=1e-6, tie_word_embeddings=False,
+)
+REFERENCE_TOK_S = 189.06  # readme.md:66: 32 requests x 64 new tokens, paged batch kernel, FP32, an unnamed CUDA GPU
 HBM_PEAK = 8.0e12  # bytes/s
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 PAGE_SIZE = 16
@@ -107,6 +123,116 @@ def time_prefill(model, cfg, tokens, repeats=3):
     return best
 
 
+def flat_config(cfg, full_layers, **more):
+    d = {"layers": cfg.num_hidden_layers, "layers_of_full_model": full_layers, "hidden": cfg.hidden_size,
+         "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+         "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "page_size": PAGE_SIZE,
+         "parallelism": "none (1 GPU)"}
+    d.update(more)
+    return d
+
+
+def reference_workload(args):
+    """The shape of the reference's benchmark (src/benchmark/generation_benchmark.cpp:259-315,
+    :430-526): 32 requests, 64-token prompts, 64 new tokens each, greedy; one warm-up run, then
+    the whole run is timed, prompts included; new tokens / wall-clock."""
+    import torch
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.engine import LLMEngine
+    from litellmengine_amd.models import random_model
+
+    cfg = Qwen3Config.from_dict(SIZES_0P6B)
+    model = random_model(cfg, seed=0, dtype=args.dtype)
+    requests, prompt_len, new_tokens = 32, 64, 64
+    pages_each = (prompt_len + new_tokens + PAGE_SIZE - 1) // PAGE_SIZE + 1
+    engine = LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_each * requests, max_requests=requests,
+                       max_tokens_per_step=requests * prompt_len, max_pages_per_request=pages_each)
+    times = []
+    for run in range(args.warmup + args.steps):
+        prompts = random_prompts(requests, prompt_len, cfg.vocab_size, 1000 + run)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = engine.generate(prompts, new_tokens)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert all(len(o) == new_tokens for o in out)
+        if run >= args.warmup:
+            times.append(dt)
+    dt = sum(times) / len(times)
+    value = requests * new_tokens / dt
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": "new tok/s of 32 requests x 64-token prompts x 64 new tokens, prompts included, Qwen3-0.6B sizes",
+        "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / REFERENCE_TOK_S, 2), "dtype": short,
+        "data": "synthetic: seeded random weights, uniform random token ids; the reference's 189.06 tok/s is FP32 "
+                "on an unnamed CUDA GPU with a real checkpoint and one text prompt",
+        "config": flat_config(cfg, SIZES_0P6B["num_hidden_layers"], model="Qwen3-0.6B sizes (random weights)",
+                              global_batch=requests, seq_len=prompt_len + new_tokens, new_tokens=new_tokens),
+    }))
+    return 0
+
+
+def mixed_workload(args):
+    """One 2048-token portion of a long prompt beside 63 decoded tokens at context 4096,
+    Qwen3-32B layer sizes: the step a serving loop runs while a prompt comes in."""
+    import torch
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.models import random_model
+
+    layers = args.layers if args.layers != SIZES["num_hidden_layers"] else SIZES_32B["num_hidden_layers"]
+    cfg = Qwen3Config.from_dict(dict(SIZES_32B, num_hidden_layers=layers))
+    model = random_model(cfg, seed=0, dtype=args.dtype)
+    decoders, context, chunk = 63, 4096, PREFILL_TOKENS
+    steps, warmup = args.steps, args.warmup
+    long_prompt = chunk * (steps + warmup)
+    pages_dec = (context + PAGE_SIZE - 1) // PAGE_SIZE + 1
+    pages_long = (long_prompt + PAGE_SIZE - 1) // PAGE_SIZE + 2
+    from litellmengine_amd.engine import LLMEngine
+
+    engine = LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_dec * decoders + pages_long,
+                       max_requests=decoders + 1, max_tokens_per_step=chunk + decoders, prefill_chunk=chunk,
+                       max_pages_per_request=max(pages_dec, pages_long))
+    prompt_len = context - (steps + warmup)
+    for p in random_prompts(decoders, prompt_len, cfg.vocab_size, 300):
+        engine.prefill(engine.add_request(p, steps + warmup + 1))
+    long_req = engine.add_request(random_prompts(1, long_prompt, cfg.vocab_size, 301)[0], 1)
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    assert long_req.finished and long_req.cached_len == long_prompt, (long_req.cached_len, long_prompt)
+    lens = [r.cached_len for r in engine.scheduler.requests.values() if r is not long_req]
+    assert all(n == context for n in lens), lens
+    tokens = chunk + decoders
+    h, d = cfg.hidden_size, cfg.head_dim
+    per_layer = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d * h + h * cfg.num_attention_heads * d
+    per_layer += 3 * h * cfg.intermediate_size
+    past_mean = chunk * (warmup + (steps - 1) / 2.0)  # keys before the timed portions, on average
+    attn = 4.0 * cfg.num_attention_heads * d * (chunk * past_mean + chunk * (chunk + 1) / 2 + decoders * context)
+    flops = (2.0 * tokens * per_layer + attn) * cfg.num_hidden_layers + 2.0 * (decoders + 1) * cfg.vocab_size * h
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": "tokens/s of a mixed step: a 2048-token prompt portion beside 63 decoded tokens at context 4096, "
+                  "Qwen3-32B sizes",
+        "value": round(tokens / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(dt * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: seeded random weights, uniform random token ids",
+        "config": flat_config(cfg, SIZES_32B["num_hidden_layers"], model="Qwen3-32B sizes (random weights)",
+                              global_batch=decoders + 1, seq_len=context, prompt_portion=chunk),
+        "roofline": {"bound": "mfma", "achieved": round(flops / dt / 1e12, 1), "peak": MFMA_PEAK[short] / 1e12,
+                     "unit": "TFLOP/s", "frac": round(flops / dt / MFMA_PEAK[short], 4)},
+    }))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -117,10 +243,22 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b"],
+                    help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
+                         "sizes, or a mixed prompt-portion + decode step at Qwen3-32B sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported")
         return 2
+    if args.workload != "decode":
+        import torch
+
+        torch.cuda.set_device(0)
+        if args.workload == "reference-0p6b":
+            args.steps, args.warmup = min(args.steps, 5), min(args.warmup, 1)
+            return reference_workload(args)
+        args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
+        return mixed_workload(args)
 
     import torch
 
