@@ -21,10 +21,12 @@
 //    32, page size a multiple of 16.  One workgroup per (request, kv head, key
 //    split); the q heads of the group (and up to 16 / group tokens) are the 16
 //    columns of v_mfma_f32_16x16x32_bf16 tiles, so every K/V byte is read once
-//    per group; the four wavefronts take every fourth 32-key step; partial
-//    (m, l, acc) of the splits are merged by the combine kernel.
+//    per group; the four wavefronts take every fourth 32-key step, their loads
+//    two steps ahead; partial (m, l, acc) of the splits are merged by the combine
+//    kernel.  In decode steps it can also do what comes before it: the q/k norm,
+//    the rotation and the write of the new K and V (FusedQKV).
 //  * mfma_prefill_kernel: same tile code, 32 rows (token, head) per wavefront,
-//    all keys up to each row's own position; the four wavefronts of a workgroup
+//    all keys up to each row's own position; the eight wavefronts of a workgroup
 //    share the K/V tiles through LDS.
 #include "common.h"
 #include <type_traits>
@@ -684,11 +686,13 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     }
 }
 
-// Requests with more than 16 rows.  grid = (row blocks of 128 x key splits, kv heads, requests);
-// each wavefront owns 32 rows.  A short portion after a long past has few row blocks: its keys
-// are then split over `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K and V^T are copied from the pages into LDS
-// once per workgroup (all 256 threads, the next tile while this one is multiplied) and every
-// wavefront reads its matrix-core operands from there: 128 rows share one pass over the keys.
+// Requests with more than 16 rows.  grid = (kv heads, row blocks x key splits, requests); a
+// workgroup takes 256 rows (128 for heads over 128 elements), each of its eight wavefronts 32
+// (16) of them.  A short portion after a long past has few row blocks: its keys are then split
+// over `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K
+// and V^T are copied from the pages into LDS once per workgroup (all threads; two tiles are on
+// their way while one is multiplied) and every wavefront reads its matrix-core operands from
+// there: the rows of a workgroup share one pass over the keys.
 //   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
 //   LDS V^T tile: [D][32 keys + 8]
 // row tiles per wavefront: two while the accumulators fit the register file

@@ -2,8 +2,9 @@
 // like the reference's Linear, src/layers/linear.cu:169-215, which calls
 // cublasSgemm).  This file holds the true 32-bit product (plain FMA, no matrix
 // cores, no reduced-precision mode; the sum over k runs in index order whatever
-// M is, so a row's result does not depend on what else is in the batch) and the
-// bfloat16 weight-streaming product of decoding.
+// M is, so a row's result does not depend on what else is in the batch), the
+// bfloat16 weight-streaming product of decoding, and its 32-bit twin (32-bit
+// operands through the 32-bit matrix instruction: products and sums in float32).
 #include "common.h"
 
 LLE_DEFINE_ERROR_STRING()
@@ -79,13 +80,13 @@ extern "C" int lle_gemm_nt_simt(const void* A, const void* B, void* C, int M, in
 // matrix that is read exactly once.  bfloat16 in, 32-bit accumulate, bfloat16 or
 // 32-bit out.  HBM-bound: the kernel is shaped to keep whole 128-byte lines of W
 // in flight from all CUs.
-//   workgroup = 16 rows of W (one matrix-core tile), 8 wavefronts split K:
-//   wavefront w takes the 64-element k steps w, w + 8, ... (neighbouring
+//   workgroup = 16 rows of W (one matrix-core tile), 16 wavefronts split K:
+//   wavefront w takes the 64-element k steps w, w + 16, ... (neighbouring
 //   wavefronts read neighbouring 128-byte pieces of the same rows);
 //   C^T tile = W tile [16 n x 64 k] . X^T [64 k x 16 m] by two
 //   v_mfma_f32_16x16x32_bf16 per 16 rows of X; lane (c = lane / 16, r = lane % 16)
 //   loads 32 contiguous bytes W[n0 + r][k0 + 16c .. + 15]; X comes from L2.
-//   The 8 partial tiles are added in LDS in wavefront order, so the sum over k
+//   The 16 partial tiles are added in LDS in wavefront order, so the sum over k
 //   has one fixed order for every M.
 // ---------------------------------------------------------------------------------
 typedef bf16_t gbf16x8 __attribute__((ext_vector_type(8)));
@@ -368,5 +369,96 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     else
         gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
             (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, fold);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------
+// The same for float32 operands: the true 32-bit path of decoding.  W is read once;
+// v_mfma_f32_16x16x4_f32 multiplies and adds in float32 (no reduced-precision mode).
+// Lane (c, r) loads 16 contiguous bytes W[n0 + r][k0 + 4c .. + 3]; its four values are the
+// k slot c of four instructions, and the X operand is laid out the same way.
+// ---------------------------------------------------------------------------------
+#define SKF_KSTEP 16
+template <int MT, int SK_WAVES, int UNROLL>
+__global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_f32_kernel(const float* __restrict__ X,
+                                                                             const float* __restrict__ W,
+                                                                             float* __restrict__ C, int M, int N, int K) {
+    __shared__ float s_acc[SK_WAVES][MT][16][17];
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const float* wp = W + min(n0 + r16, (int64_t)N - 1) * K + 4 * c;
+    // rows of X beyond M are never written back, so their lanes may read any valid row
+    const float* xp[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xp[mt] = X + (int64_t)min(16 * mt + r16, M - 1) * K + 4 * c;
+    gf32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int full_steps = K / SKF_KSTEP;
+    int ss = wave;
+    for (; ss + (UNROLL - 1) * SK_WAVES < full_steps; ss += UNROLL * SK_WAVES) {
+        gf32x4 w[UNROLL], x[UNROLL][MT];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int k0 = (ss + u * SK_WAVES) * SKF_KSTEP;
+            w[u] = *(const gf32x4*)(wp + k0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) x[u][mt] = *(const gf32x4*)(xp[mt] + k0);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[u][j], x[u][mt][j], acc[mt], 0, 0, 0);
+    }
+    // what is left of K: single steps, the last one may be partial (K is a multiple of 4)
+    const int all_steps = (K + SKF_KSTEP - 1) / SKF_KSTEP;
+    const gf32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (; ss < all_steps; ss += SK_WAVES) {
+        const int k0 = ss * SKF_KSTEP;
+        const bool in = k0 + 4 * c + 4 <= K;
+        const gf32x4 w = in ? *(const gf32x4*)(wp + k0) : zero;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const gf32x4 x = in ? *(const gf32x4*)(xp[mt] + k0) : zero;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[j], x[j], acc[mt], 0, 0, 0);
+        }
+    }
+    // lane holds C^T[n = 4c + i][m = r16]
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_acc[wave][mt][4 * c + i][r16] = acc[mt][i];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
+        const int mt = idx / 256, m = (idx / 16) % 16, n = idx % 16;
+        const int64_t row = 16 * mt + m, col = n0 + n;
+        if (row >= M || col >= N) continue;
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][mt][n][m];
+        C[row * N + col] = sum;
+    }
+}
+
+// X [M, K] and W [N, K] float32, contiguous; C [M, N] float32; 1 <= M <= 64; K a multiple of 4.
+extern "C" int lle_gemm_skinny_f32(const void* X, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 64 || K % 4 != 0 || K <= 0) return (int)hipErrorInvalidValue;
+    const int blocks = (N + 15) / 16;
+    const float* x = (const float*)X;
+    const float* w = (const float*)W;
+    float* c = (float*)C;
+    switch ((M + 15) / 16) {
+        case 1: gemm_skinny_f32_kernel<1, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
+        case 2: gemm_skinny_f32_kernel<2, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
+        case 3: gemm_skinny_f32_kernel<3, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
+        default: gemm_skinny_f32_kernel<4, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
+    }
     LLE_RETURN_LAUNCH_STATUS();
 }

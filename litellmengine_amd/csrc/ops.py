@@ -164,8 +164,9 @@ class HipOps:
         return Prenormed(xw, sums, fold.eps)
 
     def linear(self, x, weight, out_dtype=None, fold=None):
-        """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take the plain-FMA
-        kernel (a true 32-bit product).  bfloat16 operands: few rows take the
+        """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take a true 32-bit
+        product: few rows the weight-streaming kernel with the float32 matrix
+        instruction, more rows the plain-FMA kernel.  bfloat16 operands: few rows take the
         weight-streaming matrix-core kernel, more rows the library product; both
         accumulate in 32-bit and write either result type.  `x` a Prenormed or `fold`
         a NormFold: see _linear_folded."""
@@ -190,6 +191,11 @@ class HipOps:
             return torch.mm(x, weight.t()) if out_dtype == torch.bfloat16 else torch.mm(x, weight.t(), out_dtype=out_dtype)
         _need(out_dtype == torch.float32, "a float32 product has a float32 result")
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        if M <= self.SKINNY_F32_MAX_ROWS and K % 4 == 0 and not self.force_library_gemm:
+            # few rows: W streamed once, float32 matrix instruction
+            self._run("gemm", "lle_gemm_skinny_f32", [_P, _P, _P, _I, _I, _I, _P], _ptr(x), _ptr(weight), _ptr(out),
+                      M, N, K)
+            return out
         self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
@@ -197,6 +203,7 @@ class HipOps:
     # measured on MI355X: the weight-streaming kernel wins up to 8 rows for every weight, up to 16
     # rows for weights of up to 32 Mi elements; above, the library product
     SKINNY_MAX_ROWS = 8
+    SKINNY_F32_MAX_ROWS = 64  # the float32 twin: the plain-FMA kernel it replaces wastes its 64-row tiles on few rows
     SKINNY_SMALL_WEIGHT = 1 << 25
     force_library_gemm = False
 
