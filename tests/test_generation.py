@@ -204,3 +204,47 @@ def test_args_follow_the_reference():
             parse_args(["--model", "m"] + bad)
     with pytest.raises(ArgsError):
         parse_args([])
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_arrivals_small_pool_sessions_match_plain(tmp_path, seed):
+    """Requests arrive at random steps into a pool too small for all of them, some are
+    sessions that are continued once: whatever the scheduler decides (portions, preemption,
+    eviction of parked sessions), every request generates what the plain model generates
+    for its whole history, and in the end no page is held."""
+    import random
+
+    d = make_model_dir(tmp_path, "A")
+    cfg, w = plain.read_model_dir(d)
+    rng = random.Random(seed)
+    eng = cpu_engine(d, page_size=4, num_pages=14, max_requests=4, prefill_chunk=7, max_tokens_per_step=12)
+    todo = []
+    for i in range(9):
+        prompt = random_tokens(rng.randint(1, 22), 256, 100 * seed + i)
+        todo.append(dict(at=rng.randint(0, 25), prompt=prompt, new=rng.randint(1, 7), session=rng.random() < 0.4,
+                         more=random_tokens(rng.randint(1, 6), 256, 900 + 100 * seed + i), new2=rng.randint(1, 5)))
+    live, step = [], 0
+    while todo or eng.has_work() or any(x["session"] and "turn2" not in x for x in live):
+        for x in [x for x in todo if x["at"] <= step]:
+            todo.remove(x)
+            x["req"] = eng.add_request(x["prompt"], x["new"], keep_session=x["session"])
+            live.append(x)
+        for x in live:  # a finished session gets its second turn a few steps later
+            if x["session"] and "turn2" not in x and x["req"].finished and rng.random() < 0.3:
+                x["turn1"] = list(x["req"].generated)
+                eng.append_input_tokens(x["req"], x["more"], x["new2"])
+                x["turn2"] = True
+        eng.step()
+        step += 1
+        assert step < 2000
+    eng.run_until_finished()
+    assert eng.scheduler.num_preemptions + eng.scheduler.num_evictions > 0, "the pool was meant to be too small"
+    for x in live:
+        first = plain.generate_greedy(x["prompt"], w, cfg, x["new"])
+        if x["session"]:
+            assert x["turn1"] == first
+            assert x["req"].generated == plain.generate_greedy(x["prompt"] + first + x["more"], w, cfg, x["new2"])
+            eng.release_request(x["req"])
+        else:
+            assert x["req"].generated == first
+    assert all(g.pool.num_held == 0 for g in eng.cache.groups) and eng.cache.num_free_slots == 4
