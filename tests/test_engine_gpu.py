@@ -33,7 +33,7 @@ def run_cut(runner, tokens, cuts):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_cuts_match_plain(tmp_path, which, dtype):
     d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
     cfg, w = plain.read_model_dir(d)

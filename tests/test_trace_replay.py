@@ -42,7 +42,7 @@ def test_trace_cpu(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "D"])
 def test_trace_gpu(tmp_path, which, dtype):
     d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
     requests = make_requests(CONFIGS[which]["vocab_size"], seed=10)
@@ -96,7 +96,7 @@ def test_peaked_attention_trace_cpu(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["B", "C"])
+@pytest.mark.parametrize("which", ["B", "C", "D"])
 def test_peaked_attention_trace_gpu(tmp_path, which, dtype):
     d = make_model_dir(tmp_path, which, dtype=torch.bfloat16)
     factor, tol = PEAK[dtype]
