@@ -126,8 +126,8 @@ class HipOps:
     def can_fold_norm(self, rows: int, width: int, dtype) -> bool:
         """Whether an RMSNorm over `width` of a step of `rows` tokens can be done by the
         products before and after it (the weight-streaming kernel's few-rows forms)."""
-        return (dtype == torch.bfloat16 and 0 < rows <= self.SKINNY_MAX_ROWS and width % 8 == 0
-                and not self.force_library_gemm)
+        most = 16 if width <= self.SKINNY_SMALL_WIDTH else self.SKINNY_MAX_ROWS
+        return dtype == torch.bfloat16 and 0 < rows <= most and width % 8 == 0 and not self.force_library_gemm
 
     def _linear_folded(self, x, weight, fold, gated: bool):
         """The forms of the weight-streaming product around a folded norm: `x` a Prenormed
@@ -205,6 +205,7 @@ class HipOps:
     SKINNY_MAX_ROWS = 8
     SKINNY_F32_MAX_ROWS = 64  # the float32 twin: the plain-FMA kernel it replaces wastes its 64-row tiles on few rows
     SKINNY_SMALL_WEIGHT = 1 << 25
+    SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 16 rows
     force_library_gemm = False
 
     # -- attention ---------------------------------------------------------------
@@ -412,7 +413,8 @@ class HipOps:
         M, K = x.shape
         N2 = weight.shape[0]
         _need(weight.shape[1] == K and N2 % 2 == 0, f"weight {list(weight.shape)} does not fit x [{M}, {K}]")
-        if (x.dtype == torch.bfloat16 and M <= self.SKINNY_MAX_ROWS and K % 8 == 0 and not self.force_library_gemm):
+        few = M <= self.SKINNY_MAX_ROWS or (M <= 16 and N2 * K <= self.SKINNY_SMALL_WEIGHT)
+        if x.dtype == torch.bfloat16 and few and K % 8 == 0 and not self.force_library_gemm:
             out = torch.empty((M, N2 // 2), dtype=x.dtype, device=x.device)
             self._run("gemm", "lle_gemm_skinny_gated_bf16", [_P, _P, _P, _I, _I, _I, _P],
                       _ptr(x), _ptr(weight), _ptr(out), M, N2, K)
