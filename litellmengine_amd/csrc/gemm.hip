@@ -97,13 +97,13 @@ typedef float gf32x4 __attribute__((ext_vector_type(4)));
 // GATED: W holds gate rows [0, N/2) and then up rows [N/2, N); a workgroup takes 16 gate rows
 // and the 16 up rows that go with them (NT = 2) and writes silu(gate) * up, C is [M, N/2].
 //
-// The RMSNorm between two products can be folded into them (up to 16 rows).  With
+// The RMSNorm between two products can be folded into them (up to 32 rows).  With
 //   norm(h)[m][k] = h[m][k] * w[k] * r[m],  r[m] = 1 / sqrt(mean_k h[m][k]^2 + eps)
 // the factor r[m] commutes with the product that follows, so
 //   RESID (the product before the norm): its result is the delta of the residual stream; the
 //     epilogue forms h = hidden + delta in 32-bit, writes it back, writes xw = h * w as the
 //     next product's input, and leaves the sum of h^2 over its 16 columns per row in
-//     ss_part[16][workgroups];
+//     ss_part[16 MT][workgroups];
 //   SCALED (the product after the norm): adds up the parts, and multiplies its rows by r[m].
 struct NormFold {
     float* hidden;          // RESID: residual stream [M, N], read and written
@@ -123,15 +123,16 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
                                                                          const bf16_t* __restrict__ W,
                                                                          TC* __restrict__ C, int M, int N, int K,
                                                                          NormFold fold) {
-    static_assert(!(RESID || SCALED) || MT == 1, "the norm is folded for up to 16 rows");
+    static_assert(!(RESID || SCALED) || MT <= 2, "the norm is folded for up to 32 rows");
     // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
-    __shared__ float s_inv[16];
+    __shared__ float s_inv[16 * MT];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
-    // SCALED: wavefront m adds up the parts of row m.  The first parts are asked for now and
-    // added after the products, so that their way from memory is not waited for up front.
-    static_assert(!SCALED || SK_WAVES == 16, "one wavefront per row of the norm");
-    constexpr int EARLY_PARTS = GATED ? 0 : 4;  // the gated form has no registers to spare for them
+    // SCALED: wavefront w adds up the parts of the rows w, w + 16.  With one tile of rows the
+    // first parts are asked for now and added after the products, so that their way from
+    // memory is not waited for up front.
+    static_assert(!SCALED || SK_WAVES == 16, "one wavefront per row of a tile of the norm");
+    constexpr int EARLY_PARTS = (GATED || MT > 1) ? 0 : 4;  // where registers are to spare for them
     float early[EARLY_PARTS + 1];
     if (SCALED) {
 #pragma unroll
@@ -144,13 +145,18 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
     const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
     // RESID: thread (m, n) of the first 256 owns element [m][n0 + n]; what it needs of the
     // residual stream and of the norm weight is asked for now and has arrived by the epilogue
-    float resid_h = 0.f, resid_w = 0.f;
+    float resid_h[MT], resid_w = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) resid_h[mt] = 0.f;
     if (RESID && threadIdx.x < 256) {
-        const int m = threadIdx.x / 16;
         const int64_t col = n0 + threadIdx.x % 16;
-        if (m < M && col < N) {
-            resid_h = fold.hidden[(int64_t)m * N + col];
+        if (col < N) {
             resid_w = load_as_f32(fold.weight, col, fold.weight_dtype);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = 16 * mt + threadIdx.x / 16;
+                if (m < M) resid_h[mt] = fold.hidden[(int64_t)m * N + col];
+            }
         }
     }
     const bf16_t* wp[NT];
@@ -225,13 +231,17 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
         }
     }
     if (SCALED) {
-        float part = 0.f;
 #pragma unroll
-        for (int i = 0; i < EARLY_PARTS; ++i) part += early[i];
-        for (int b = lane + LLE_WAVE * EARLY_PARTS; b < fold.parts; b += LLE_WAVE)
-            part += fold.ss_in[(int64_t)wave * fold.parts + b];
-        part = wave_sum(part);
-        if (lane == 0) s_inv[wave] = 1.0f / sqrtf(part / (float)K + fold.eps);
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = 16 * mt + wave;
+            float part = 0.f;
+#pragma unroll
+            for (int i = 0; i < EARLY_PARTS; ++i) part += early[i];
+            for (int b = lane + LLE_WAVE * EARLY_PARTS; b < fold.parts; b += LLE_WAVE)
+                part += fold.ss_in[(int64_t)m * fold.parts + b];
+            part = wave_sum(part);
+            if (lane == 0) s_inv[m] = 1.0f / sqrtf(part / (float)K + fold.eps);
+        }
     }
     // lane holds C^T[n = 4c + i][m = r16]
 #pragma unroll
@@ -253,30 +263,34 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
                 u += s_acc[w][NT - 1][mt][n][m];
             }
             if (SCALED) {
-                g *= s_inv[m];
-                u *= s_inv[m];
+                g *= s_inv[16 * mt + m];
+                u *= s_inv[16 * mt + m];
             }
             C[row * (N / 2) + col] = from_f32<TC>(g / (1.0f + expf(-g)) * u);
         }
         return;
     }
-    if (RESID) {  // NT = MT = 1
+    if (RESID) {  // NT = 1
         if (threadIdx.x < 256) {
-            const int m = threadIdx.x / 16, n = threadIdx.x % 16;
+            const int n = threadIdx.x % 16;
             const int64_t col = n0 + n;
-            float sq = 0.f;
-            if (m < M && col < N) {
-                float sum = 0.f;
 #pragma unroll
-                for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][0][n][m];
-                const float h = resid_h + sum;
-                fold.hidden[(int64_t)m * N + col] = h;
-                fold.xw[(int64_t)m * N + col] = (bf16_t)(h * resid_w);
-                sq = h * h;
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m16 = threadIdx.x / 16, m = 16 * mt + m16;
+                float sq = 0.f;
+                if (m < M && col < N) {
+                    float sum = 0.f;
+#pragma unroll
+                    for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][mt][n][m16];
+                    const float h = resid_h[mt] + sum;
+                    fold.hidden[(int64_t)m * N + col] = h;
+                    fold.xw[(int64_t)m * N + col] = (bf16_t)(h * resid_w);
+                    sq = h * h;
+                }
+#pragma unroll
+                for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, LLE_WAVE);
+                if (n == 0) fold.ss_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
             }
-#pragma unroll
-            for (int o = 1; o < 16; o <<= 1) sq += __shfl_xor(sq, o, LLE_WAVE);
-            if (n == 0) fold.ss_out[(int64_t)m * gridDim.x + blockIdx.x] = sq;
         }
         return;
     }
@@ -287,7 +301,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][nt][mt][n][m];
-        if (SCALED) sum *= s_inv[m];
+        if (SCALED) sum *= s_inv[16 * mt + m];
         C[row * N + col] = from_f32<TC>(sum);
     }
 }
@@ -335,40 +349,52 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
 
 // The product BEFORE a folded norm: delta = X W^T [M, N] is added into `hidden` (float32 [M, N],
 // in place), xw = hidden * norm_weight goes to `xw` (bfloat16 [M, N]) and the sums of squares of
-// the new hidden over each workgroup's 16 columns to ss_part [16][(N + 15) / 16].  1 <= M <= 16.
+// the new hidden over each workgroup's 16 columns to ss_part [16 or 32][(N + 15) / 16] (32 rows
+// when M > 16).  1 <= M <= 32.
 extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hidden, const void* norm_weight,
                                           int weight_dtype, void* xw, void* ss_part, int M, int N, int K,
                                           hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K % 8 != 0 || K <= 0) return (int)hipErrorInvalidValue;
+    if (M > 32 || K % 8 != 0 || K <= 0) return (int)hipErrorInvalidValue;
     NormFold fold = {};
     fold.hidden = (float*)hidden;
     fold.weight = norm_weight;
     fold.weight_dtype = weight_dtype;
     fold.xw = (bf16_t*)xw;
     fold.ss_out = (float*)ss_part;
-    gemm_skinny_kernel<1, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
-        (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
+    if (M <= 16)
+        gemm_skinny_kernel<1, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
+    else
+        gemm_skinny_kernel<2, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
 // The product AFTER a folded norm: X is the xw of lle_gemm_skinny_resid_bf16 and ss_part its
-// 16 x `parts` sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).  gated != 0:
-// W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.  1 <= M <= 16.
+// (16 or 32) x `parts` sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).
+// gated != 0: W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.
+// 1 <= M <= 32.
 extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C, const void* ss_part, int parts,
                                            float eps, int M, int N, int K, int gated, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (M > 16 || K % 8 != 0 || K <= 0 || parts <= 0 || (gated && N % 2 != 0)) return (int)hipErrorInvalidValue;
+    if (M > 32 || K % 8 != 0 || K <= 0 || parts <= 0 || (gated && N % 2 != 0)) return (int)hipErrorInvalidValue;
     NormFold fold = {};
     fold.ss_in = (const float*)ss_part;
     fold.parts = parts;
     fold.eps = eps;
-    if (gated)
-        gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
-            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, fold);
+    const bf16_t* x = (const bf16_t*)X;
+    const bf16_t* w = (const bf16_t*)W;
+    bf16_t* c = (bf16_t*)C;
+    const int threads = 16 * LLE_WAVE;
+    if (gated && M <= 16)
+        gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
+    else if (gated)
+        gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
+    else if (M <= 16)
+        gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
     else
-        gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
-            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, fold);
+        gemm_skinny_kernel<2, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
     LLE_RETURN_LAUNCH_STATUS();
 }
 

@@ -126,7 +126,7 @@ class HipOps:
     def can_fold_norm(self, rows: int, width: int, dtype) -> bool:
         """Whether an RMSNorm over `width` of a step of `rows` tokens can be done by the
         products before and after it (the weight-streaming kernel's few-rows forms)."""
-        most = 16 if width <= self.SKINNY_SMALL_WIDTH else self.SKINNY_MAX_ROWS
+        most = 32 if width <= self.SKINNY_SMALL_WIDTH else self.SKINNY_MAX_ROWS
         return dtype == torch.bfloat16 and 0 < rows <= most and width % 8 == 0 and not self.force_library_gemm
 
     def _linear_folded(self, x, weight, fold, gated: bool):
@@ -140,12 +140,14 @@ class HipOps:
         M, K = xin.shape
         N = weight.shape[0]
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
-        _need(self.can_fold_norm(M, K, xin.dtype), f"a norm cannot be folded into a product of {M} rows of {K}")
+        _need(K % 8 == 0, f"the weight-streaming product needs a multiple of 8 columns, not {K}")
         _need(pre is None or fold is None, "a product takes a Prenormed or makes one, not both")
         if pre is not None:
+            _need(self.can_fold_norm(M, K, xin.dtype), f"a norm over {K} cannot be folded for {M} rows")
             _dev(pre.sums, "sums", torch.float32)
             parts = pre.sums.shape[1]
-            _need(pre.sums.shape == (16, parts) and pre.xw.shape[1] == K, "sums of squares do not fit")
+            _need(pre.sums.shape == (16 if M <= 16 else 32, parts) and pre.xw.shape[1] == K,
+                  "sums of squares do not fit")
             _need(not gated or N % 2 == 0, "a gated weight has an even number of rows")
             out = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=xin.device)
             self._run("gemm", "lle_gemm_skinny_scaled_bf16", [_P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
@@ -155,9 +157,9 @@ class HipOps:
         _dev(fold.weight, "norm weight")
         _need(not gated and fold.hidden.shape == (M, N) and fold.weight.shape == (N,),
               f"residual stream {list(fold.hidden.shape)} does not fit a product [{M}, {N}]")
-        _need(self.can_fold_norm(M, N, xin.dtype), f"a norm over {N} cannot be folded")
+        _need(self.can_fold_norm(M, N, xin.dtype), f"a norm over {N} cannot be folded for {M} rows")
         xw = torch.empty((M, N), dtype=torch.bfloat16, device=xin.device)
-        sums = torch.empty((16, (N + 15) // 16), dtype=torch.float32, device=xin.device)
+        sums = torch.empty((16 if M <= 16 else 32, (N + 15) // 16), dtype=torch.float32, device=xin.device)
         self._run("gemm", "lle_gemm_skinny_resid_bf16", [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
                   _ptr(xin), _ptr(weight), _ptr(fold.hidden), _ptr(fold.weight), dtype_code(fold.weight.dtype),
                   _ptr(xw), _ptr(sums), M, N, K)
@@ -205,7 +207,7 @@ class HipOps:
     SKINNY_MAX_ROWS = 8
     SKINNY_F32_MAX_ROWS = 64  # the float32 twin: the plain-FMA kernel it replaces wastes its 64-row tiles on few rows
     SKINNY_SMALL_WEIGHT = 1 << 25
-    SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 16 rows
+    SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 32 rows
     force_library_gemm = False
 
     # -- attention ---------------------------------------------------------------
@@ -413,7 +415,7 @@ class HipOps:
         M, K = x.shape
         N2 = weight.shape[0]
         _need(weight.shape[1] == K and N2 % 2 == 0, f"weight {list(weight.shape)} does not fit x [{M}, {K}]")
-        few = M <= self.SKINNY_MAX_ROWS or (M <= 16 and N2 * K <= self.SKINNY_SMALL_WEIGHT)
+        few = M <= self.SKINNY_MAX_ROWS or (M <= 32 and N2 * K <= self.SKINNY_SMALL_WEIGHT)
         if x.dtype == torch.bfloat16 and few and K % 8 == 0 and not self.force_library_gemm:
             out = torch.empty((M, N2 // 2), dtype=x.dtype, device=x.device)
             self._run("gemm", "lle_gemm_skinny_gated_bf16", [_P, _P, _P, _I, _I, _I, _P],

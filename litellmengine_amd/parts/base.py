@@ -75,7 +75,7 @@ class Prenormed:
     `ops.linear` and `ops.gate_up_silu` take one, and each value is used once."""
 
     xw: torch.Tensor  # [N, width], hidden * norm weight, activation type
-    sums: torch.Tensor  # float32 [16, parts]: row m's sums of squares of hidden over column ranges
+    sums: torch.Tensor  # float32 [16 or 32, parts]: row m's sums of squares of hidden over column ranges
     eps: float
 
 

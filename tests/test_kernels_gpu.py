@@ -100,7 +100,8 @@ def test_gate_up_silu(dtype, M, I, K):
 
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,H,K,N", [(1, 64, 40, 48), (3, 136, 72, 100), (8, 4096, 1024, 512), (5, 1000, 64, 30),
-                                     (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70)])
+                                     (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70), (32, 1024, 2048, 3072),
+                                     (17, 72, 40, 22), (29, 2048, 512, 128)])
 def test_norm_folded_into_products(wdtype, M, H, K, N):
     """RMSNorm between two products, done by them: the first adds its result into the
     residual stream and leaves hidden * w and sums of squares, the second (plain or
@@ -109,7 +110,7 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
     from litellmengine_amd.parts import NormFold
 
     o = ops()
-    assert o.can_fold_norm(M, H, torch.bfloat16) and not o.can_fold_norm(17, H, torch.bfloat16)
+    assert o.can_fold_norm(M, H, torch.bfloat16) and not o.can_fold_norm(33, H, torch.bfloat16)
     assert o.can_fold_norm(9, H, torch.bfloat16) == (H <= 2048), "more than 8 rows only for narrow models"
     assert not o.can_fold_norm(M, H, torch.float32) and not o.can_fold_norm(M, H + 4, torch.bfloat16)
     a = rnd((M, K), torch.bfloat16, 31)
@@ -124,7 +125,7 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         pre = o.linear(a, w1, fold=NormFold(h, nw, eps))
         want_h = hidden.double() + a.double() @ w1.double().t()
         assert (h.double() - want_h).abs().max() < 1e-4 * max(1.0, want_h.abs().max().item())
-        assert pre.sums.shape == (16, (H + 15) // 16)
+        assert pre.sums.shape == (16 if M <= 16 else 32, (H + 15) // 16)
         ss = pre.sums.double().sum(1)[:M]
         assert torch.allclose(ss, (want_h ** 2).sum(1), rtol=1e-5)
         normed = want_h * torch.rsqrt((want_h ** 2).mean(1, keepdim=True) + eps) * nw.double()
