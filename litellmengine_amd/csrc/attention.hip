@@ -26,8 +26,8 @@
 //    kernel.  In decode steps it can also do what comes before it: the q/k norm,
 //    the rotation and the write of the new K and V (FusedQKV).
 //  * mfma_prefill_kernel: same tile code, 32 rows (token, head) per wavefront,
-//    all keys up to each row's own position; the eight wavefronts of a workgroup
-//    share the K/V tiles through LDS.
+//    all keys up to each row's own position; the four wavefronts of a workgroup
+//    share the K/V tiles through LDS, two workgroups share a CU.
 #include "common.h"
 #include <type_traits>
 
@@ -687,8 +687,9 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 }
 
 // Requests with more than 16 rows.  grid = (kv heads, row blocks x key splits, requests); a
-// workgroup takes 256 rows (128 for heads over 128 elements), each of its eight wavefronts 32
-// (16) of them.  A short portion after a long past has few row blocks: its keys are then split
+// workgroup takes 128 rows (64 for heads over 128 elements), each of its four wavefronts 32
+// (16) of them; two workgroups fit a CU (256 registers a lane each), which measured faster
+// than one of twice the size: a heavy and a light row block then share a CU.  A short portion after a long past has few row blocks: its keys are then split
 // over `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K
 // and V^T are copied from the pages into LDS once per workgroup (all threads; two tiles are on
 // their way while one is multiplied) and every wavefront reads its matrix-core operands from
@@ -697,19 +698,20 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 //   LDS V^T tile: [D][32 keys + 8]
 // row tiles per wavefront: two while the accumulators fit the register file
 #ifndef PRE_WAVES
-#define PRE_WAVES 8
+#define PRE_WAVES 4
 #endif
 #ifndef PRE_RT_MAX
 #define PRE_RT_MAX 2
 #endif
 #define PRE_RT_OF(DK) ((DK) <= 4 ? PRE_RT_MAX : 1)
 template <int DK>
-__global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
+// (heads over 192 elements need more than the 256 registers a lane that two workgroups a CU leave)
+__global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int ws_stride, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages,
-    int window, float scale_log2) {
+    int window, float scale_log2, int complement_order) {
     constexpr int D = DK * 32;
     constexpr int PRE_RT = PRE_RT_OF(DK);
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
@@ -726,10 +728,15 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     const int q_len = cu_tokens[s + 1] - q_start;
     const int nrows = q_len * G;
     if (nrows <= 16) return;  // the decode kernel's
-    // the last rows see the most keys: they are started first
+    // The last rows see the most keys: they are started first.  When the whole launch is
+    // resident at once (two workgroups a CU) the order is: the heavy half of the row blocks,
+    // heaviest first, then the light half, lightest first, so that the two workgroups that
+    // come to share a CU (launch positions j and j + half) add up to about the same work.
     const int row_blocks = gridDim.y / nsplit;
     const int split = blockIdx.y / row_blocks;
-    const int block_row0 = (row_blocks - 1 - blockIdx.y % row_blocks) * PRE_ROWS;
+    const int yb = blockIdx.y % row_blocks, heavy_blocks = (row_blocks + 1) / 2;
+    const int block_row0 =
+        (complement_order && yb >= heavy_blocks ? yb - heavy_blocks : row_blocks - 1 - yb) * PRE_ROWS;
     if (block_row0 >= nrows) return;
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
@@ -895,6 +902,19 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, 1) void mfma_prefill_kernel(
     }
 }
 
+// CUs of the current device (asked once per device)
+static int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
 template <int DK, bool FUSED>
 static int launch_decode(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_tables, const int32_t* seq_slots,
                          const int32_t* cu_tokens, const int32_t* kv_lens, bf16_t* out, float* ws_o, float* ws_ml,
@@ -946,9 +966,10 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
         constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT_OF(DK);
         const int rows = max_q_len * G;
         const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
+        const int64_t workgroups = (int64_t)nkv * blocks * nsplit_prefill * S;
         mfma_prefill_kernel<DK><<<dim3(nkv, blocks * nsplit_prefill, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
             q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill, nq,
-            nkv, P, page_stride, max_pages, window, scale_log2);
+            nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0);
     }
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
         mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(

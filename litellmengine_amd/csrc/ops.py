@@ -376,7 +376,7 @@ class HipOps:
                        max_kv_len: int, window: int) -> int:
         """Key splits of the prompt-portion kernel: 1 unless the portions are so short that
         their row blocks alone leave most of the chip idle (a tail of a prompt after a long past)."""
-        rows_per_block = 256 if head_dim <= 128 else 128
+        rows_per_block = 128 if head_dim <= 128 else 64
         blocks = ((max_q_len * group + rows_per_block - 1) // rows_per_block) * num_kv_heads * max(1, num_seqs)
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
         steps = (span + 31) // 32
