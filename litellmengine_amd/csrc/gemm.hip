@@ -63,6 +63,83 @@ __global__ __launch_bounds__(256) void gemm_nt_simt_kernel(const TA* __restrict_
     }
 }
 
+// The same product through the 32-bit matrix instruction (v_mfma_f32_16x16x4_f32: float32
+// operands, products and sums; no reduced-precision mode), for many rows: 64 x 64 tiles, four
+// wavefronts of 32 x 32 each, k in steps of 16 through LDS.  Lane (c, r) reads 16 bytes
+// T[row r][4c .. 4c + 3] of a tile; its four values are the k slot c of four instructions, for
+// both operands alike.  The sum over k runs in the same order for every tile, whatever M is.
+// K must be a multiple of 4 (16-byte loads).
+typedef float mf32x4 __attribute__((ext_vector_type(4)));
+#define GM_LD (GT_BK + 4)  // row stride in LDS: 80 bytes, 16-byte reads of 16 rows fall into different banks
+__global__ __launch_bounds__(256) void gemm_nt_mfma_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                               float* __restrict__ C, int M, int N, int K,
+                                                               int64_t lda, int64_t ldb, int64_t ldc) {
+    __shared__ __attribute__((aligned(16))) float As[GT_BM * GM_LD];
+    __shared__ __attribute__((aligned(16))) float Bs[GT_BN * GM_LD];
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    const int64_t m0 = (int64_t)blockIdx.y * GT_BM, n0 = (int64_t)blockIdx.x * GT_BN;
+    const int wm = (wave / 2) * 32, wn = (wave % 2) * 32;  // this wavefront's corner in the tile
+    // the copy into LDS: thread -> (row of the tile, 4 consecutive k)
+    const int lr = threadIdx.x / 4, lk = (threadIdx.x % 4) * 4;
+    const bool a_row = m0 + lr < M, b_row = n0 + lr < N;
+    const float* ap = A + (m0 + lr) * lda + lk;
+    const float* bp = B + (n0 + lr) * ldb + lk;
+    const mf32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    mf32x4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = zero;
+
+    for (int k0 = 0; k0 < K; k0 += GT_BK) {
+        const bool kin = k0 + lk < K;  // K is a multiple of 4: a piece is inside or outside as a whole
+        const mf32x4 av = (a_row && kin) ? *(const mf32x4*)(ap + k0) : zero;
+        const mf32x4 bv = (b_row && kin) ? *(const mf32x4*)(bp + k0) : zero;
+        __syncthreads();  // the tiles of the step before are read
+        *(mf32x4*)(As + lr * GM_LD + lk) = av;
+        *(mf32x4*)(Bs + lr * GM_LD + lk) = bv;
+        __syncthreads();
+        mf32x4 a[2], b[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) a[i] = *(const mf32x4*)(As + (wm + 16 * i + r16) * GM_LD + 4 * c);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) b[j] = *(const mf32x4*)(Bs + (wn + 16 * j + r16) * GM_LD + 4 * c);
+        // C^T tile [n][m] = B tile . A tile^T: lane holds C^T[n = 4c + e][m = r16], as in the skinny kernels
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(b[j][e], a[i][e], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int64_t m = m0 + wm + 16 * i + r16;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t n = n0 + wn + 16 * j + 4 * c + e;
+                if (n < N) C[m * ldc + n] = acc[i][j][e];
+            }
+    }
+}
+
+// float32 in, float32 out; K a multiple of 4, rows 16-byte aligned (lda, ldb multiples of 4)
+extern "C" int lle_gemm_nt_mfma_f32(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda,
+                                    int64_t ldb, int64_t ldc, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || K % 4 != 0 || lda % 4 != 0 || ldb % 4 != 0) return (int)hipErrorInvalidValue;
+    dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM);
+    if (grid.y > 65535) return (int)hipErrorInvalidValue;
+    gemm_nt_mfma_f32_kernel<<<grid, 256, 0, stream>>>((const float*)A, (const float*)B, (float*)C, M, N, K, lda, ldb,
+                                                       ldc);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
 // float32 in, float32 out (in_dtype and out_dtype must say so)
 extern "C" int lle_gemm_nt_simt(const void* A, const void* B, void* C, int M, int N, int K, int64_t lda,
                                 int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, hipStream_t stream) {

@@ -167,8 +167,8 @@ class HipOps:
 
     def linear(self, x, weight, out_dtype=None, fold=None):
         """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take a true 32-bit
-        product: few rows the weight-streaming kernel with the float32 matrix
-        instruction, more rows the plain-FMA kernel.  bfloat16 operands: few rows take the
+        product: few rows the weight-streaming kernel, more rows a tiled kernel, both
+        with the float32 matrix instruction; the plain-FMA kernel where K is no multiple of 4.  bfloat16 operands: few rows take the
         weight-streaming matrix-core kernel, more rows the library product; both
         accumulate in 32-bit and write either result type.  `x` a Prenormed or `fold`
         a NormFold: see _linear_folded."""
@@ -198,6 +198,11 @@ class HipOps:
             self._run("gemm", "lle_gemm_skinny_f32", [_P, _P, _P, _I, _I, _I, _P], _ptr(x), _ptr(weight), _ptr(out),
                       M, N, K)
             return out
+        if K % 4 == 0 and not self.force_simt_gemm:
+            # many rows: 64 x 64 tiles through the float32 matrix instruction
+            self._run("gemm", "lle_gemm_nt_mfma_f32", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _P],
+                      _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N)
+            return out
         self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
@@ -209,6 +214,7 @@ class HipOps:
     SKINNY_SMALL_WEIGHT = 1 << 25
     SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 32 rows
     force_library_gemm = False
+    force_simt_gemm = False  # tests flip this to reach the plain-FMA kernel at sizes the matrix instruction takes
 
     # -- attention ---------------------------------------------------------------
     def rope_table(self, positions, inv_freq) -> torch.Tensor:

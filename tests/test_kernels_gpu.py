@@ -169,6 +169,26 @@ def test_linear(in_dtype, out_dtype, M, N, K):
     assert (got.double() - want).abs().max() < lim * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 64, 16), (130, 96, 72), (300, 513, 1024), (2048, 1000, 136), (77, 151, 4)])
+def test_linear_float32_many_rows(M, N, K):
+    """The tiled float32 kernel (float32 matrix instruction) and the plain-FMA kernel it stands beside."""
+    x = rnd((M, K), torch.float32, 61)
+    w = rnd((N, K), torch.float32, 62, 0.05)
+    want = x.double() @ w.double().t()
+    o = ops()
+    got = o.linear(x, w)
+    o.force_simt_gemm = True
+    try:
+        plain = o.linear(x, w)
+    finally:
+        o.force_simt_gemm = False
+    lim = 1e-5 * max(1.0, want.abs().max().item())
+    assert (got.double() - want).abs().max() < lim and (plain.double() - want).abs().max() < lim
+    # a row's result does not depend on what else is in the batch
+    part = o.linear(x[40:].contiguous(), w)
+    assert torch.equal(part, got[40:])
+
+
 def test_linear_reference_vector():
     # tests/test_linear.cpp:63-78: X 2x3, W 4x3
     x = torch.tensor([[1.0, 2, 3], [4, 5, 6]]).cuda()
