@@ -248,3 +248,28 @@ def test_random_arrivals_small_pool_sessions_match_plain(tmp_path, seed):
         else:
             assert x["req"].generated == first
     assert all(g.pool.num_held == 0 for g in eng.cache.groups) and eng.cache.num_free_slots == 4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sessions_on_the_gpu(tmp_path, dtype):
+    """Two sessions and a plain request on the GPU (the sizes whose small bfloat16 steps take the
+    fused decode paths): turns continued from the cache generate what the plain model generates
+    for the whole history; nothing is held after release."""
+    d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    model = load_model(d, dtype)
+    eng = LLMEngine(model, page_size=16, num_pages=24, max_requests=3, prefill_chunk=20)
+    firsts = [random_tokens(n, 419, 70 + i) for i, n in enumerate((37, 9, 50))]
+    mores = [random_tokens(n, 419, 80 + i) for i, n in enumerate((11, 3))]
+    reqs = [eng.add_request(p, 6, keep_session=i < 2) for i, p in enumerate(firsts)]
+    eng.run_until_finished()
+    gen1 = [plain.generate_greedy(p, w, cfg, 6) for p in firsts]
+    assert [r.generated for r in reqs] == gen1
+    for r, more in zip(reqs[:2], mores):
+        eng.append_input_tokens(r, more, 5)
+    eng.run_until_finished()
+    for r, p, g, more in zip(reqs[:2], firsts, gen1, mores):
+        assert r.generated == plain.generate_greedy(p + g + more, w, cfg, 5)
+        eng.release_request(r)
+    assert all(g.pool.num_held == 0 for g in eng.cache.groups)
