@@ -696,6 +696,8 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 // there: the rows of a workgroup share one pass over the keys.
 //   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
 //   LDS V^T tile: [D][32 keys + 8]
+// Heads of 128 elements skip the registers: global_load_lds_dwordx4 writes the tiles into LDS
+// directly (three unpadded, XOR-swizzled buffers; see the DMA branch of the kernel).
 // row tiles per wavefront: two while the accumulators fit the register file
 #ifndef PRE_WAVES
 #define PRE_WAVES 4
@@ -718,7 +720,9 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     constexpr int KROW = D + 8;       // elements per key row in LDS
     constexpr int VROW = KSTEP + 8;   // elements per value-element row in LDS: 16-byte pieces stay aligned
     constexpr int TILE = KSTEP * KROW + D * VROW;
-    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * TILE];
+    constexpr bool DMA = DK == 4 && PRE_WAVES == 4;  // tiles straight into LDS (measured 4-5 % faster)
+    constexpr int DTILE = 2 * KSTEP * D;  // elements of a tile without padding: K [32][D], then V^T [D][32]
+    __shared__ __attribute__((aligned(16))) bf16_t lds[DMA ? 3 * DTILE : 2 * TILE];
 
     // the kv head varies fastest: workgroups go to the eight dies in turn, each die has an L2 of
     // its own, and this way a die sees the K/V of few heads, which the row blocks of a head share
@@ -865,13 +869,81 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         __syncthreads();
     };
 
-    fetch(std::integral_constant<int, 0>{});  // tile first_step
-    fetch(std::integral_constant<int, 1>{});  // tile first_step + 1
-    stash(0, std::integral_constant<int, 0>{});
-    __syncthreads();
-    for (int step = first_step; step < end_step; step += 2) {
-        one_step(step, 0, std::integral_constant<int, 1>{});
-        one_step(step + 1, 1, std::integral_constant<int, 0>{});  // multiplies nothing past my_end
+    if constexpr (DMA) {
+        // Tiles go from the pages straight into LDS (no registers, no stores by the wavefronts):
+        // a wavefront's load writes 1 KB of LDS in lane order (M0 holds where), so the tiles have
+        // no padding, and the 16-byte pieces of a row are XOR-swizzled instead, by which piece
+        // each lane fetches.  The loads are written in assembly so that the waits are ours: the
+        // compiler, seeing such a load, waits for ALL outstanding loads before every barrier.
+        // vmcnt counts them in issue order, so "at most the 4 newest outstanding" means that
+        // every tile requested before the last one has landed, whatever else was issued.
+        //   K  [32 keys][16 pieces]: logical piece p of key j at piece p ^ (j % 16)
+        //   V^T [D][4 pieces]:       logical piece p (keys 8p..8p+7) of element e at piece p ^ ((e / 4) % 4)
+        // Three buffers: tile N is multiplied, N + 1 has landed or lands, N + 2 is requested.
+        const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)lds;
+        const int tid = threadIdx.x;
+        int64_t kd_thread[2], vd_thread[2];
+        int vd_half[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int q = tid + 256 * i;
+            const int key = q / 16, pk = q % 16;  // K: this half's key (i = half), physical piece
+            kd_thread[i] = (int64_t)(key % 16) * D + ((pk ^ (key % 16)) * 8);
+            const int e = q / 4, pv = q % 4;
+            const int lp = pv ^ ((e / 4) % 4);  // logical piece: keys 8 lp .. 8 lp + 7 of the step
+            vd_half[i] = lp / 2;
+            vd_thread[i] = (int64_t)e * P + (lp % 2) * 8;
+        }
+        auto dma = [&](int buf) {
+            const bf16_t* half0 = kv_layer + (int64_t)page_id[0] * page_stride;
+            const bf16_t* half1 = kv_layer + (int64_t)page_id[1] * page_stride;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const bf16_t* kp = (i ? half1 : half0) + k_head + (int64_t)(i ? page_off[1] : page_off[0]) * D + kd_thread[i];
+                const bf16_t* vp = (vd_half[i] ? half1 : half0) + v_head + (vd_half[i] ? page_off[1] : page_off[0]) + vd_thread[i];
+                const unsigned kdst = __builtin_amdgcn_readfirstlane(lds_base + 2 * (buf * DTILE + (wave * 64 + 256 * i) * 8));
+                const unsigned vdst = kdst + 2 * KSTEP * D;
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(kdst), "v"(kp) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(vdst), "v"(vp) : "memory", "m0");
+            }
+            lookup();
+        };
+        const int kx[2] = {KEY_OF_ROW(r16, 0), KEY_OF_ROW(r16, 1)};
+        const int vsw = (r16 / 4) % 4;
+        auto dma_step = [&](int step, int buf, int next_buf) {
+            dma(next_buf);  // tile step + 2
+            if (step >= my_first && step < my_end) {
+                const bf16_t* kt = lds + buf * DTILE;
+                const bf16_t* vt = kt + KSTEP * D;
+                tile_step<DK, PRE_RT>(
+                    st, row,
+                    [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ (kx[x] % 16)) * 8)); },
+                    [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * KSTEP + ((c ^ vsw) * 8)); },
+                    step * KSTEP, scale_log2);
+            }
+            // the four loads just issued may stay in flight; the tile before them has landed
+            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+        };
+        dma(0);  // tile first_step
+        dma(1);  // tile first_step + 1
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        for (int step = first_step; step < end_step; step += 3) {
+            dma_step(step, 0, 2);
+            dma_step(step + 1, 1, 0);
+            dma_step(step + 2, 2, 1);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land after the workgroup has gone
+    } else {
+        fetch(std::integral_constant<int, 0>{});  // tile first_step
+        fetch(std::integral_constant<int, 1>{});  // tile first_step + 1
+        stash(0, std::integral_constant<int, 0>{});
+        __syncthreads();
+        for (int step = first_step; step < end_step; step += 2) {
+            one_step(step, 0, std::integral_constant<int, 1>{});
+            one_step(step + 1, 1, std::integral_constant<int, 0>{});  // multiplies nothing past my_end
+        }
     }
     finish_rows<DK, PRE_RT>(st);
 #pragma unroll
