@@ -204,10 +204,12 @@ __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&
     // The rows of Q are waited for here, once.  Left pending, their first use lies inside the
     // key loop, where the wait for them also waits for the K/V loads just issued for a later
     // step: the loop would run at the latency of memory.
+    if (LOAD_Q) {
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+        for (int t = 0; t < RT; ++t)
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) asm volatile("" : "+v"(st.qv[t][ks]));
+            for (int ks = 0; ks < DK; ++ks) asm volatile("" : "+v"(st.qv[t][ks]));
+    }
 }
 
 // One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key
@@ -326,11 +328,15 @@ struct StepOperands {
 // meet again): the loop runs an even number of steps, loads past the end go to a page that is
 // there, and the CALLER has limited the rows' `pos` to the last key of step_end - 1, so that a
 // step past the end is masked out whole.
-template <int DK, int RT, bool LOAD_Q = true>
+// `before_keys()` runs when the first table lookup is on its way and no operand is asked for yet:
+// what the caller loads there travels beside the lookup, what it stores there is stored before
+// this wavefront reads any key.  `after_first_loads()` runs once the first two steps are asked for.
+template <int DK, int RT, bool LOAD_Q = true, typename BeforeKeys, typename AfterFirstLoads>
 __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT],
                                             const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ table,
                                             int kvh, int nkv, int P, int64_t page_stride, int step_begin,
-                                            int step_end, int step_stride, int lo_min, int hi, float scale_log2) {
+                                            int step_end, int step_stride, int lo_min, int hi, float scale_log2,
+                                            BeforeKeys before_keys, AfterFirstLoads after_first_loads) {
     constexpr int D = DK * 32;
     const int lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
@@ -383,8 +389,10 @@ __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo 
     };
     StepOperands<DK> even, odd;
     lookup();
+    before_keys();
     load(even);
     load(odd);
+    after_first_loads();
     for (int step = step_begin; step < step_end; step += 2 * step_stride) {
         multiply(even, step);
         load(even);
@@ -425,63 +433,94 @@ struct FusedQKV {
     int write_kv;
 };
 
-__device__ __forceinline__ void load_weights8(const void* w, int e, int dtype, float (&out)[8]) {
+// Eight consecutive norm weights (float32 or bfloat16) as they lie in memory; what they mean is
+// decided by weights8_as_f32 AFTER the loads have met again.  (Converted inside the branch that
+// knows the type, every load would be waited for on the spot, one memory latency each.)
+struct RawWeights8 {
+    uint32_t bits[8];  // bfloat16: the first four words hold the eight values
+};
+__device__ __forceinline__ void load_raw_weights8(const void* w, int e, int dtype, RawWeights8& out) {
     if (dtype == LLE_F32) {
-        const float4 a = *(const float4*)((const float*)w + e), b = *(const float4*)((const float*)w + e + 4);
-        out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+        const uint4 a = *(const uint4*)((const float*)w + e), b = *(const uint4*)((const float*)w + e + 4);
+        out.bits[0] = a.x, out.bits[1] = a.y, out.bits[2] = a.z, out.bits[3] = a.w;
+        out.bits[4] = b.x, out.bits[5] = b.y, out.bits[6] = b.z, out.bits[7] = b.w;
     } else {
-        const bf16x8 v = *(const bf16x8*)((const bf16_t*)w + e);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
+        const uint4 a = *(const uint4*)((const bf16_t*)w + e);
+        out.bits[0] = a.x, out.bits[1] = a.y, out.bits[2] = a.z, out.bits[3] = a.w;
+        out.bits[4] = out.bits[5] = out.bits[6] = out.bits[7] = 0u;
     }
+}
+__device__ __forceinline__ float weights8_as_f32(const RawWeights8& raw, int i, bool is_f32) {
+    const uint32_t word = raw.bits[i / 2];
+    const uint32_t as_bf16 = (i % 2) ? (word & 0xffff0000u) : (word << 16);
+    return __uint_as_float(is_f32 ? raw.bits[i] : as_bf16);
+}
+// one weight: the word it lies in (a bfloat16 value in the low half), read by weight_as_f32
+__device__ __forceinline__ uint32_t load_raw_weight(const void* w, int e, int dtype) {
+    if (dtype == LLE_F32) return ((const uint32_t*)w)[e];
+    return ((const uint16_t*)w)[e];
+}
+__device__ __forceinline__ float weight_as_f32(uint32_t raw, bool is_f32) {
+    return __uint_as_float(is_f32 ? raw : raw << 16);
 }
 
 // Q^T operands of the lane's row from the raw projection: norm over the head (its 4 * DK * 8
 // elements sit in the four lanes r16 + 16 c), weight, rotation.  Element 32 ks + 8 c + i and its
 // partner D / 2 further on are both in this lane (DK is even).  Rounded to bfloat16 as the
-// separate kernel rounds q.
+// separate kernel rounds q.  Everything is ASKED FOR in one go (load) and worked on later
+// (finish): a load that followed the arithmetic on another would cost the memory's latency again.
 template <int DK>
-__device__ __forceinline__ void fused_q_row(bf16x8 (&qv)[DK], const bf16_t* src, const FusedQKV& f, int64_t tok) {
+struct FusedQRow {
     static_assert(DK % 2 == 0, "rotation partners lie in one lane only for an even number of 32-element blocks");
-    constexpr int D = DK * 32;
-    const int c = (threadIdx.x % LLE_WAVE) / 16;
-    float x[DK][8];
+    bf16x8 raw[DK];
+    RawWeights8 w[DK];
+    float4 tab[DK / 2][4];  // cos, sin of element 2 i, then of 2 i + 1
+
+    // `src`: the head of a row that exists (lanes of rows that do not exist read another row's and drop it)
+    __device__ __forceinline__ void load(const bf16_t* src, const FusedQKV& f, int64_t tok) {
+        constexpr int D = DK * 32;
+        const int c = (threadIdx.x % LLE_WAVE) / 16;
 #pragma unroll
-    for (int ks = 0; ks < DK; ++ks) {
-        bf16x8 v;
-        if (src) {
-            v = *(const bf16x8*)(src + 32 * ks + 8 * c);
-        } else {
+        for (int ks = 0; ks < DK; ++ks) raw[ks] = *(const bf16x8*)(src + 32 * ks + 8 * c);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = (bf16_t)0.0f;
+        for (int ks = 0; ks < DK / 2; ++ks) {
+            const float4* t = (const float4*)(f.cos_sin + (tok * (D / 2) + 32 * ks + 8 * c) * 2);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) tab[ks][i] = t[i];
         }
+        if (f.q_weight) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[ks][i] = (float)v[i];
+            for (int ks = 0; ks < DK; ++ks) load_raw_weights8(f.q_weight, 32 * ks + 8 * c, f.weight_dtype, w[ks]);
+        }
     }
-    if (f.q_weight) {
-        float ss = 0.f;
+
+    __device__ __forceinline__ void finish(bf16x8 (&qv)[DK], bool exists, const FusedQKV& f) const {
+        constexpr int D = DK * 32;
+        float x[DK][8];
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) ss += x[ks][i] * x[ks][i];
-        ss += __shfl_xor(ss, 16, LLE_WAVE);
-        ss += __shfl_xor(ss, 32, LLE_WAVE);
-        const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+            for (int i = 0; i < 8; ++i) x[ks][i] = exists ? (float)raw[ks][i] : 0.f;
+        if (f.q_weight) {
+            float ss = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) {
-            float w[8];
-            load_weights8(f.q_weight, 32 * ks + 8 * c, f.weight_dtype, w);
+            for (int ks = 0; ks < DK; ++ks)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[ks][i] = x[ks][i] * inv * w[i];
+                for (int i = 0; i < 8; ++i) ss += x[ks][i] * x[ks][i];
+            ss += __shfl_xor(ss, 16, LLE_WAVE);
+            ss += __shfl_xor(ss, 32, LLE_WAVE);
+            const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+            const bool is_f32 = f.weight_dtype == LLE_F32;
+#pragma unroll
+            for (int ks = 0; ks < DK; ++ks)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[ks][i] = x[ks][i] * inv * weights8_as_f32(w[ks], i, is_f32);
         }
-    }
-    if (src) {
 #pragma unroll
         for (int ks = 0; ks < DK / 2; ++ks) {
-            const float4* tab = (const float4*)(f.cos_sin + (tok * (D / 2) + 32 * ks + 8 * c) * 2);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float4 t = tab[i];  // cos, sin of element 2 i, then of 2 i + 1
+                const float4 t = tab[ks][i];
                 const float a0 = x[ks][2 * i], b0 = x[ks + DK / 2][2 * i];
                 const float a1 = x[ks][2 * i + 1], b1 = x[ks + DK / 2][2 * i + 1];
                 x[ks][2 * i] = a0 * t.x - b0 * t.y;
@@ -490,58 +529,70 @@ __device__ __forceinline__ void fused_q_row(bf16x8 (&qv)[DK], const bf16_t* src,
                 x[ks + DK / 2][2 * i + 1] = b1 * t.z + a1 * t.w;
             }
         }
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qv[ks][i] = (bf16_t)x[ks][i];
     }
-#pragma unroll
-    for (int ks = 0; ks < DK; ++ks)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) qv[ks][i] = (bf16_t)x[ks][i];
-}
+};
 
 // One wavefront: K (norm, weight, rotation) and V of token `tok`, kv head `kvh`, into the pages.
-// Lane l takes elements l, l + 64, ... < D / 2 and their partners D / 2 further on.
+// Lane l takes elements l, l + 64, ... < D / 2 and their partners D / 2 further on.  All loads
+// are asked for before anything waits for one of them.
 template <int DK>
 __device__ __forceinline__ void fused_kv_write(const FusedQKV& f, int64_t tok, int kvh, int nq, int nkv,
                                                bf16_t* kv_layer, int P, int64_t page_stride) {
     constexpr int D = DK * 32, HALF = D / 2, PER = (HALF + LLE_WAVE - 1) / LLE_WAVE;
     const int lane = threadIdx.x % LLE_WAVE;
     const int slot = f.slots[tok];
-    if (slot < 0) return;
-    const int page = slot / P, off = slot - page * P;
     const bf16_t* ksrc = f.qkv + (tok * (nq + 2 * nkv) + nq + kvh) * D;
     const bf16_t* vsrc = ksrc + (int64_t)nkv * D;
+    float lo[PER], hi[PER];
+    uint32_t wlo[PER], whi[PER];
+    bf16_t vlo[PER], vhi[PER];
+    float2 tab[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int e = min(lane + LLE_WAVE * j, HALF - 1);  // lanes past the half read its last element and drop it
+        lo[j] = (float)ksrc[e];
+        hi[j] = (float)ksrc[e + HALF];
+        vlo[j] = vsrc[e];
+        vhi[j] = vsrc[e + HALF];
+        tab[j] = *(const float2*)(f.cos_sin + (tok * HALF + e) * 2);
+        wlo[j] = whi[j] = 0x3f80u;  // 1 as bfloat16
+    }
+    const bool is_f32 = f.k_weight && f.weight_dtype == LLE_F32;
+    if (f.k_weight) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int e = min(lane + LLE_WAVE * j, HALF - 1);
+            wlo[j] = load_raw_weight(f.k_weight, e, f.weight_dtype);
+            whi[j] = load_raw_weight(f.k_weight, e + HALF, f.weight_dtype);
+        }
+    }
+    if (slot < 0) return;
+    const int page = slot / P, off = slot - page * P;
     bf16_t* page_base = kv_layer + (int64_t)page * page_stride;
     bf16_t* kdst = page_base + ((int64_t)kvh * P + off) * D;
     bf16_t* vdst = page_base + ((int64_t)nkv + kvh) * P * D + off;  // element e at vdst[e * P]
-    float lo[PER], hi[PER];
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        const int e = lane + LLE_WAVE * j;
-        lo[j] = e < HALF ? (float)ksrc[e] : 0.f;
-        hi[j] = e < HALF ? (float)ksrc[e + HALF] : 0.f;
-        ss += lo[j] * lo[j] + hi[j] * hi[j];
-    }
+    float inv = 1.f;
     if (f.k_weight) {
-        ss = wave_sum(ss);
-        const float inv = 1.0f / sqrtf(ss / (float)D + f.eps);
+        float ss = 0.f;
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            const int e = lane + LLE_WAVE * j;
-            if (e < HALF) {
-                lo[j] = lo[j] * inv * load_as_f32(f.k_weight, e, f.weight_dtype);
-                hi[j] = hi[j] * inv * load_as_f32(f.k_weight, e + HALF, f.weight_dtype);
-            }
-        }
+        for (int j = 0; j < PER; ++j)
+            if (lane + LLE_WAVE * j < HALF) ss += lo[j] * lo[j] + hi[j] * hi[j];
+        ss = wave_sum(ss);
+        inv = 1.0f / sqrtf(ss / (float)D + f.eps);
     }
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int e = lane + LLE_WAVE * j;
         if (e < HALF) {
-            const float2 t = *(const float2*)(f.cos_sin + (tok * HALF + e) * 2);
-            kdst[e] = (bf16_t)(lo[j] * t.x - hi[j] * t.y);
-            kdst[e + HALF] = (bf16_t)(hi[j] * t.x + lo[j] * t.y);
-            vdst[(int64_t)e * P] = vsrc[e];
-            vdst[(int64_t)(e + HALF) * P] = vsrc[e + HALF];
+            const float a = lo[j] * inv * weight_as_f32(wlo[j], is_f32), b = hi[j] * inv * weight_as_f32(whi[j], is_f32);
+            kdst[e] = (bf16_t)(a * tab[j].x - b * tab[j].y);
+            kdst[e + HALF] = (bf16_t)(b * tab[j].x + a * tab[j].y);
+            vdst[(int64_t)e * P] = vlo[j];
+            vdst[(int64_t)(e + HALF) * P] = vhi[j];
         }
     }
 }
@@ -564,17 +615,26 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     float* s_m = smem + DEC_WAVES * 16 * D;
     float* s_l = s_m + DEC_WAVES * 16;
 
+    // A launch of this kernel is short, and what it waits for before its first key counts.  All
+    // arguments are read here in one go, and so is all that is known of the request: read where
+    // they are first used, each group would cost a round trip to memory of its own.
+    // (The four tables that are read with scalar loads stay out of the statement: a pointer that
+    // it has seen counts as written to, and loads through it would become vector loads.)
+    asm volatile("" ::"s"(q), "s"(kv_layer), "s"(out), "s"(ws_o), "s"(ws_ml), "s"(ws_stride), "s"(nq), "s"(nkv), "s"(P),
+                 "s"(page_stride), "s"(max_pages), "s"(window), "s"(scale_log2), "s"(fused.qkv), "s"(fused.slots),
+                 "s"(fused.q_weight), "s"(fused.k_weight), "s"(fused.weight_dtype), "s"(fused.cos_sin),
+                 "s"(fused.eps), "s"(fused.write_kv));
     const int s = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, nsplit = gridDim.z;
     const int G = nq / nkv;
-    const int q_start = cu_tokens[s];
-    const int q_len = cu_tokens[s + 1] - q_start;
+    const int q_start = cu_tokens[s], q_end = cu_tokens[s + 1], kv_len = kv_lens[s], seq_slot = seq_slots[s];
+    asm volatile("" ::"s"(q_start), "s"(q_end), "s"(kv_len), "s"(seq_slot));
+    const int q_len = q_end - q_start;
     const int nrows = q_len * G;
-    if (nrows > 16) return;  // the prefill kernel's
-    const int kv_len = kv_lens[s];
+    if (nrows > 16 || nrows <= 0) return;  // the prefill kernel's, or nothing to do
     const int past = kv_len - q_len;
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
+    const int32_t* table = block_tables + (int64_t)seq_slot * max_pages;
 
     // FUSED: q is made here from the projection; the row's pointer only says that the row exists
     RowInfo row[1] = {make_row(FUSED ? fused.qkv : q, r16, nrows, G, q_start, past, nq, kvh, D, window)};
@@ -586,32 +646,37 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int se = min(last + 1, sb + per_split);
     // keys of later splits are not this workgroup's: attend_rows may run a step past `se`
     row[0].pos = min(row[0].pos, se * KSTEP - 1);
-    if (FUSED) {
-        // The new keys and values of this head that lie in this workgroup's share of the steps
-        // go into the pages first; no other workgroup reads them in this launch, and this one
-        // reads them only after the barrier, by which the stores are done.
-        if (fused.write_kv) {
-            for (int t = wave; t < q_len; t += DEC_WAVES) {
-                const int step_of = (past + t) / KSTEP;
-                if (step_of >= sb && step_of < se)
-                    fused_kv_write<DK>(fused, (int64_t)q_start + t, kvh, nq, nkv, kv_layer, P, page_stride);
-            }
-        }
-        __syncthreads();
-    }
 
     RowState<DK, 1> st;
     if constexpr (FUSED) {
-        const bf16_t* src = nullptr;
-        int64_t tok = 0;
-        if (r16 < nrows) {
-            tok = (int64_t)q_start + r16 / G;
-            src = fused.qkv + (tok * (nq + 2 * nkv) + kvh * G + r16 % G) * D;
-        }
-        fused_q_row<DK>(st.qv[0], src, fused, tok);
+        // The raw q row, its rotation table and the norm weights are asked for while the table
+        // lookup is on its way.  A new token's K and V go into the pages by the hand of the
+        // wavefront that multiplies the token's step (step sb + wave, + DEC_WAVES, ...): it
+        // stores them before it asks for any key, no other wavefront of this launch needs them
+        // (one that runs a step past its share masks that step out whole), and so no barrier
+        // stands between the write and the keys.
+        FusedQRow<DK> qrow;
+        const int rr = r16 < nrows ? r16 : 0;
+        const int64_t tok = (int64_t)q_start + rr / G;
+        attend_rows<DK, 1, false>(
+            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi, scale_log2,
+            [&]() {
+                qrow.load(fused.qkv + (tok * (nq + 2 * nkv) + kvh * G + rr % G) * D, fused, tok);
+                if (fused.write_kv) {
+                    for (int t = 0; t < q_len; ++t) {
+                        const int step_of = (past + t) / KSTEP;
+                        if (step_of >= sb && step_of < se && (step_of - sb) % DEC_WAVES == wave)
+                            fused_kv_write<DK>(fused, (int64_t)q_start + t, kvh, nq, nkv, kv_layer, P, page_stride);
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                }
+            },
+            [&]() { qrow.finish(st.qv[0], r16 < nrows, fused); });
+    } else {
+        attend_rows<DK, 1, true>(
+            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi, scale_log2,
+            []() {}, []() {});
     }
-    attend_rows<DK, 1, !FUSED>(st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min,
-                               hi, scale_log2);
 
     // merge the wavefronts (rows that do not exist are not worth the LDS traffic)
     if (r16 < nrows) {
@@ -678,11 +743,28 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     const float big = wave_max(m);
     const float f = exp2f(m - big);  // 0 for lanes without a split (l = 0 there anyway)
     const float den = wave_sum(l * f);
+    // every lane needs every split's factor, also those of lanes that have no element below
+    __shared__ float s_f[LLE_WAVE];
+    s_f[lane] = f;
+    __syncthreads();
+    // A lane takes two neighbouring elements; the partial sums of eight splits are loaded
+    // together (one load after the other would pay the memory's latency once per split).
     const float* o = ws_o + head_row * ws_stride * D;
-    for (int e = lane; e < D; e += LLE_WAVE) {
-        float num = 0.f;
-        for (int k = 0; k < nsplit; ++k) num += o[(int64_t)k * D + e] * __shfl(f, k, LLE_WAVE);
-        out[head_row * D + e] = (bf16_t)(num / den);
+    for (int e = 2 * lane; e < D; e += 2 * LLE_WAVE) {
+        float2 num = {0.f, 0.f};
+        for (int k0 = 0; k0 < nsplit; k0 += 8) {
+            float2 part[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) part[j] = *(const float2*)(o + (int64_t)min(k0 + j, nsplit - 1) * D + e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float fk = k0 + j < nsplit ? s_f[k0 + j] : 0.f;
+                num.x += part[j].x * fk;
+                num.y += part[j].y * fk;
+            }
+        }
+        out[head_row * D + e] = (bf16_t)(num.x / den);
+        out[head_row * D + e + 1] = (bf16_t)(num.y / den);
     }
 }
 

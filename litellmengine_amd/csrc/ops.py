@@ -371,10 +371,10 @@ class HipOps:
 
     force_generic_attention = False  # tests flip this to compare the two families of kernels
     force_separate_rope = False      # tests flip this to compare the fused decode step with its two halves
-    # measured on MI355X: about one workgroup per CU and at least 16 32-key steps (four per
+    # measured on MI355X: about one workgroup per CU and at least 8 32-key steps (two per
     # wavefront) per split are best; more splits cost more in partial results than they gain
     DECODE_TARGET_BLOCKS = 256
-    DECODE_MIN_STEPS_PER_SPLIT = 16
+    DECODE_MIN_STEPS_PER_SPLIT = 8
 
     PREFILL_MIN_STEPS_PER_SPLIT = 8
 
