@@ -204,37 +204,44 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
     // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
     __shared__ float s_inv[16 * MT];
+    // A launch is short: what stands between its start and its first load of W counts.  All
+    // arguments are read in one go (read where they are first used, each group costs a round
+    // trip of its own), and the small loads beside W (parts of the norm's sums, residual
+    // stream, norm weight) are asked for without a condition around them, so that nothing
+    // waits for them before the loads of W are on their way.
+    asm volatile("" ::"s"(X), "s"(W), "s"(C), "s"(M), "s"(N), "s"(K), "s"(fold.hidden), "s"(fold.weight),
+                 "s"(fold.weight_dtype), "s"(fold.xw), "s"(fold.ss_out), "s"(fold.ss_in), "s"(fold.parts),
+                 "s"(fold.eps));
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     // SCALED: wavefront w adds up the parts of the rows w, w + 16.  With one tile of rows the
-    // first parts are asked for now and added after the products, so that their way from
-    // memory is not waited for up front.
+    // first parts are asked for now and added after the products.
     static_assert(!SCALED || SK_WAVES == 16, "one wavefront per row of a tile of the norm");
-    constexpr int EARLY_PARTS = (GATED || MT > 1) ? 0 : 4;  // where registers are to spare for them
+    constexpr int EARLY_PARTS = (GATED || MT > 1) ? 0 : 4;  // the gated form measured faster without them
     float early[EARLY_PARTS + 1];
     if (SCALED) {
 #pragma unroll
-        for (int i = 0; i < EARLY_PARTS; ++i) {
-            const int b = lane + LLE_WAVE * i;
-            early[i] = b < fold.parts ? fold.ss_in[(int64_t)wave * fold.parts + b] : 0.f;
-        }
+        for (int i = 0; i < EARLY_PARTS; ++i)  // past the parts: the last one again, dropped below
+            early[i] = fold.ss_in[(int64_t)wave * fold.parts + min(lane + LLE_WAVE * i, fold.parts - 1)];
     }
     const int c = lane / 16, r16 = lane % 16;
     const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
     // RESID: thread (m, n) of the first 256 owns element [m][n0 + n]; what it needs of the
     // residual stream and of the norm weight is asked for now and has arrived by the epilogue
-    float resid_h[MT], resid_w = 0.f;
+    // (all threads ask, for places that are there; the bits of the weight are read as they lie
+    // and interpreted in the epilogue)
+    float resid_h[MT];
+    uint32_t resid_w = 0;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) resid_h[mt] = 0.f;
-    if (RESID && threadIdx.x < 256) {
-        const int64_t col = n0 + threadIdx.x % 16;
-        if (col < N) {
-            resid_w = load_as_f32(fold.weight, col, fold.weight_dtype);
+    if (RESID) {
+        const int64_t col = min(n0 + threadIdx.x % 16, (int64_t)N - 1);
+        if (fold.weight_dtype == LLE_F32)
+            resid_w = ((const uint32_t*)fold.weight)[col];
+        else
+            resid_w = ((const uint16_t*)fold.weight)[col];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int m = 16 * mt + threadIdx.x / 16;
-                if (m < M) resid_h[mt] = fold.hidden[(int64_t)m * N + col];
-            }
-        }
+        for (int mt = 0; mt < MT; ++mt)
+            resid_h[mt] = fold.hidden[(int64_t)min(16 * mt + (int)(threadIdx.x / 16) % 16, M - 1) * N + col];
     }
     const bf16_t* wp[NT];
 #pragma unroll
@@ -313,9 +320,16 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
             const int m = 16 * mt + wave;
             float part = 0.f;
 #pragma unroll
-            for (int i = 0; i < EARLY_PARTS; ++i) part += early[i];
-            for (int b = lane + LLE_WAVE * EARLY_PARTS; b < fold.parts; b += LLE_WAVE)
-                part += fold.ss_in[(int64_t)m * fold.parts + b];
+            for (int i = 0; i < EARLY_PARTS; ++i) part += lane + LLE_WAVE * i < fold.parts ? early[i] : 0.f;
+            // what is left: four loads at a time (one after the other would each pay the way from memory)
+            const float* in = fold.ss_in + (int64_t)m * fold.parts;
+            for (int b = lane + LLE_WAVE * EARLY_PARTS; b < fold.parts; b += 4 * LLE_WAVE) {
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] = in[min(b + i * LLE_WAVE, fold.parts - 1)];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) part += b + i * LLE_WAVE < fold.parts ? v[i] : 0.f;
+            }
             part = wave_sum(part);
             if (lane == 0) s_inv[m] = 1.0f / sqrtf(part / (float)K + fold.eps);
         }
@@ -361,7 +375,8 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
                     for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][mt][n][m16];
                     const float h = resid_h[mt] + sum;
                     fold.hidden[(int64_t)m * N + col] = h;
-                    fold.xw[(int64_t)m * N + col] = (bf16_t)(h * resid_w);
+                    fold.xw[(int64_t)m * N + col] =
+                        (bf16_t)(h * __uint_as_float(fold.weight_dtype == LLE_F32 ? resid_w : resid_w << 16));
                     sq = h * h;
                 }
 #pragma unroll
@@ -381,6 +396,177 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
         if (SCALED) sum *= s_inv[16 * mt + m];
         C[row * N + col] = from_f32<TC>(sum);
     }
+}
+
+// ---------------------------------------------------------------------------------
+// The gated product as a STREAM, for K = 64 * 16 * XS (XS steps per wavefront, XS even,
+// all of X that a wavefront needs held in registers) and up to 16 rows.  One workgroup
+// per CU stays and walks over the tiles of W (tile t, t + workgroups, ...).  A wavefront
+// keeps two sets of W operands: while one is multiplied the loads of the next are on
+// their way, also across the end of a tile, where the partial tiles are added up in LDS
+// and written out.  X is read once per workgroup instead of once per tile, and the sums
+// of the folded norm are added up once per workgroup.
+// ---------------------------------------------------------------------------------
+template <bool SCALED, int XS>
+__global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(const bf16_t* __restrict__ X,
+                                                                             const bf16_t* __restrict__ W,
+                                                                             bf16_t* __restrict__ C, int M, int N, int K,
+                                                                             NormFold fold) {
+    static_assert(XS % 4 == 0, "sets of two steps of W are multiplied in pairs");
+    constexpr int WAVES = 16;
+    __shared__ float s_acc[2][WAVES][2][16][17];  // tiles take the two halves in turn: one barrier a tile
+    __shared__ float s_inv[16];
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    const int rows = N / 2;
+    const int tiles = (rows + 15) / 16;
+
+    // a set: two 64-element steps of the gate tile and of the up tile
+    struct Set {
+        gbf16x8 g0[2], g1[2], u0[2], u1[2];
+    };
+    // the load cursor: tile and step of the set that is asked for next
+    int load_tile = blockIdx.x, load_step = 0;
+    const bf16_t* wp = nullptr;
+    auto aim = [&]() {
+        wp = W + (int64_t)min(16 * load_tile + r16, rows - 1) * K + 16 * c + wave * SK_KSTEP;
+    };
+    auto load = [&](Set& set) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const bf16_t* g = wp + (load_step + i) * (WAVES * SK_KSTEP);
+            const bf16_t* u = g + (int64_t)rows * K;
+            set.g0[i] = *(const gbf16x8*)g;
+            set.g1[i] = *(const gbf16x8*)(g + 8);
+            set.u0[i] = *(const gbf16x8*)u;
+            set.u1[i] = *(const gbf16x8*)(u + 8);
+        }
+        load_step += 2;
+        if (load_step == XS) {
+            load_step = 0;
+            load_tile += gridDim.x;
+            aim();
+        }
+    };
+    Set a, b;
+    aim();
+    load(a);
+    // rows of X beyond M are never written back, so their lanes may read any valid row
+    gbf16x8 x0[XS], x1[XS];
+    {
+        const bf16_t* xp = X + (int64_t)min(r16, M - 1) * K + 16 * c + wave * SK_KSTEP;
+#pragma unroll
+        for (int j = 0; j < XS; ++j) {
+            x0[j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP));
+            x1[j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP) + 8);
+        }
+    }
+    if (SCALED) {
+        // the row factors of the folded norm: wavefront w adds up the parts of row w, four loads at a time
+        const float* in = fold.ss_in + (int64_t)wave * fold.parts;
+        float part = 0.f;
+        for (int p0 = lane; p0 < fold.parts; p0 += 4 * LLE_WAVE) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = in[min(p0 + i * LLE_WAVE, fold.parts - 1)];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part += p0 + i * LLE_WAVE < fold.parts ? v[i] : 0.f;
+        }
+        part = wave_sum(part);
+        if (lane == 0) s_inv[wave] = 1.0f / sqrtf(part / (float)K + fold.eps);
+    }
+    gf32x4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const Set& set, int j) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g0[i], x0[j + i], acc_g, 0, 0, 0);
+            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g1[i], x1[j + i], acc_g, 0, 0, 0);
+            acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u0[i], x0[j + i], acc_u, 0, 0, 0);
+            acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u1[i], x1[j + i], acc_u, 0, 0, 0);
+        }
+    };
+    int half = 0;
+    auto finish_tile = [&](int tile) {
+        // lane holds C^T[n = 4c + i][m = r16]
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s_acc[half][wave][0][4 * c + i][r16] = acc_g[i];
+            s_acc[half][wave][1][4 * c + i][r16] = acc_u[i];
+        }
+        acc_g = acc_u = gf32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            const int m = threadIdx.x / 16, n = threadIdx.x % 16;
+            const int64_t col = (int64_t)tile * 16 + n;
+            if (m < M && col < rows) {
+                float g = 0.f, u = 0.f;
+#pragma unroll
+                for (int w = 0; w < WAVES; ++w) {
+                    g += s_acc[half][w][0][n][m];
+                    u += s_acc[half][w][1][n][m];
+                }
+                if (SCALED) {
+                    g *= s_inv[m];
+                    u *= s_inv[m];
+                }
+                C[(int64_t)m * rows + col] = (bf16_t)(g / (1.0f + expf(-g)) * u);
+            }
+        }
+        // The other half is written next; this one again only after the next tile's barrier,
+        // which the threads that are still adding here have then passed.
+        half ^= 1;
+    };
+
+    int tile = blockIdx.x;
+    for (; tile + (int)gridDim.x < tiles; tile += gridDim.x) {  // every tile of this workgroup but its last
+#pragma unroll
+        for (int j = 0; j < XS; j += 4) {
+            load(b);
+            multiply(a, j);
+            load(a);  // after the tile's last set: the first of the next tile
+            multiply(b, j + 2);
+        }
+        finish_tile(tile);
+    }
+    if (tile < tiles) {  // the last one asks for nothing beyond itself
+#pragma unroll
+        for (int j = 0; j < XS; j += 4) {
+            load(b);
+            multiply(a, j);
+            if (j + 4 < XS) load(a);
+            multiply(b, j + 2);
+        }
+        finish_tile(tile);
+    }
+}
+
+// CUs of the current device (asked once per device)
+static int gemm_compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// The streaming kernel takes the product when its shape is the one it is built for (K = 4096,
+// up to 16 rows) and every workgroup gets at least two tiles and all of them about the same
+// number (one a CU; a last round that most CUs sit out would cost more than the stream gains).
+template <bool SCALED>
+static bool launch_gated_stream(const bf16_t* X, const bf16_t* W, bf16_t* C, int M, int N, int K, const NormFold& fold,
+                                hipStream_t stream) {
+    constexpr int XS = 4;
+    if (M > 16 || K != SK_KSTEP * 16 * XS) return false;
+    const int tiles = (N / 2 + 15) / 16;
+    const int blocks = gemm_compute_units();
+    const int rounds = (tiles + blocks - 1) / blocks;
+    if (rounds < 2 || (int64_t)rounds * blocks * 9 > (int64_t)tiles * 10) return false;
+    gemm_gated_stream_kernel<SCALED, XS><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, fold);
+    return true;
 }
 
 template <typename TC, int NT, bool GATED>
@@ -421,6 +607,8 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
                                           hipStream_t stream) {
     if (M <= 0 || N2 <= 0) return 0;
     if (M > 32 || K % 8 != 0 || K <= 0 || N2 % 2 != 0) return (int)hipErrorInvalidValue;
+    if (launch_gated_stream<false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, NormFold{}, stream))
+        LLE_RETURN_LAUNCH_STATUS();
     return launch_skinny<bf16_t, 2, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, stream);
 }
 
@@ -464,7 +652,8 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     const bf16_t* w = (const bf16_t*)W;
     bf16_t* c = (bf16_t*)C;
     const int threads = 16 * LLE_WAVE;
-    if (gated && M <= 16)
+    if (gated && launch_gated_stream<true>(x, w, c, M, N, K, fold, stream)) {
+    } else if (gated && M <= 16)
         gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
     else if (gated)
         gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);

@@ -86,7 +86,8 @@ def test_silu_mul(dtype, I):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,I,K", [(1, 128, 64), (5, 200, 96), (8, 12288, 4096), (8, 136, 80), (9, 100, 72), (40, 64, 48)])
+@pytest.mark.parametrize("M,I,K", [(1, 128, 64), (5, 200, 96), (8, 12288, 4096), (8, 136, 80), (9, 100, 72), (40, 64, 48),
+                                   (3, 12277, 4096), (1, 8189, 4096)])
 def test_gate_up_silu(dtype, M, I, K):
     x = rnd((M, K), dtype, 21, 2.0)
     w = rnd((2 * I, K), dtype, 22, 0.1)
@@ -100,6 +101,7 @@ def test_gate_up_silu(dtype, M, I, K):
 
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,H,K,N", [(1, 64, 40, 48), (3, 136, 72, 100), (8, 4096, 1024, 512), (5, 1000, 64, 30),
+                                     (6, 4096, 256, 8189), (1, 4096, 128, 12288),
                                      (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70), (32, 1024, 2048, 3072),
                                      (17, 72, 40, 22), (29, 2048, 512, 128)])
 def test_norm_folded_into_products(wdtype, M, H, K, N):
