@@ -399,52 +399,66 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 }
 
 // ---------------------------------------------------------------------------------
-// The gated product as a STREAM, for K = 64 * 16 * XS (XS steps per wavefront, XS even,
-// all of X that a wavefront needs held in registers) and up to 16 rows.  One workgroup
-// per CU stays and walks over the tiles of W (tile t, t + workgroups, ...).  A wavefront
-// keeps two sets of W operands: while one is multiplied the loads of the next are on
-// their way, also across the end of a tile, where the partial tiles are added up in LDS
-// and written out.  X is read once per workgroup instead of once per tile, and the sums
-// of the folded norm are added up once per workgroup.
+// The product as a STREAM, for K = 64 * 16 * XS (XS steps per wavefront, all of X that a
+// wavefront needs held in registers) and up to 16 rows of X; plain or gated, with or
+// without the row factors of a folded norm.
+// How fast a CU reads is bounded by the loads it can have on their way, so the chip is
+// fastest when every CU has the same share of W.  There is one workgroup per CU, and it
+// takes `share` rows of W (share = rows / CUs, rounded up) in tiles of 16, the last of
+// which may be lower: tile t of all workgroups together is one block of consecutive rows
+// (the memory channels see what they see of a plain sweep over W), of which workgroup b
+// takes the b-th piece.  The lanes of a tile that is not full read its last row again,
+// which costs no traffic.  A wavefront keeps two sets of W operands: while one is multiplied
+// the loads of the next are on their way, also across the end of a tile, where the
+// partial tiles are added up in LDS and written out.  X is read once per workgroup
+// instead of once per tile, and the sums of the folded norm are added up once.
 // ---------------------------------------------------------------------------------
-template <bool SCALED, int XS>
-__global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(const bf16_t* __restrict__ X,
-                                                                             const bf16_t* __restrict__ W,
-                                                                             bf16_t* __restrict__ C, int M, int N, int K,
-                                                                             NormFold fold) {
+template <bool GATED, bool SCALED, int XS>
+__global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X,
+                                                                              const bf16_t* __restrict__ W,
+                                                                              bf16_t* __restrict__ C, int M, int N, int K,
+                                                                              int share, NormFold fold) {
     static_assert(XS % 4 == 0, "sets of two steps of W are multiplied in pairs");
     constexpr int WAVES = 16;
-    __shared__ float s_acc[2][WAVES][2][16][17];  // tiles take the two halves in turn: one barrier a tile
+    constexpr int NT = GATED ? 2 : 1;
+    __shared__ float s_acc[2][WAVES][NT][16][17];  // tiles take the two halves in turn: one barrier a tile
     __shared__ float s_inv[16];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int rows = N / 2;
-    const int tiles = (rows + 15) / 16;
+    const int rows = GATED ? N / 2 : N;
+    const int tiles = (share + 15) / 16;
+    // rows [tile_begin(t), tile_end(t)) of this workgroup's tile t; none where W ends before them
+    auto tile_begin = [&](int t) { return (int)gridDim.x * 16 * t + (int)blockIdx.x * min(16, share - 16 * t); };
+    auto tile_end = [&](int t) { return min(rows, tile_begin(t) + min(16, share - 16 * t)); };
 
-    // a set: two 64-element steps of the gate tile and of the up tile
+    // a set: two 64-element steps of the tile (and of the up tile that goes with a gate tile)
     struct Set {
         gbf16x8 g0[2], g1[2], u0[2], u1[2];
     };
     // the load cursor: tile and step of the set that is asked for next
-    int load_tile = blockIdx.x, load_step = 0;
+    int load_tile = 0, load_step = 0;
     const bf16_t* wp = nullptr;
     auto aim = [&]() {
-        wp = W + (int64_t)min(16 * load_tile + r16, rows - 1) * K + 16 * c + wave * SK_KSTEP;
+        const int t = min(load_tile, tiles - 1);
+        const int row = max(0, min(tile_begin(t) + r16, tile_end(t) - 1));  // a tile without rows reads rows that are there
+        wp = W + (int64_t)row * K + 16 * c + wave * SK_KSTEP;
     };
     auto load = [&](Set& set) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const bf16_t* g = wp + (load_step + i) * (WAVES * SK_KSTEP);
-            const bf16_t* u = g + (int64_t)rows * K;
             set.g0[i] = *(const gbf16x8*)g;
             set.g1[i] = *(const gbf16x8*)(g + 8);
-            set.u0[i] = *(const gbf16x8*)u;
-            set.u1[i] = *(const gbf16x8*)(u + 8);
+            if (GATED) {
+                const bf16_t* u = g + (int64_t)rows * K;
+                set.u0[i] = *(const gbf16x8*)u;
+                set.u1[i] = *(const gbf16x8*)(u + 8);
+            }
         }
         load_step += 2;
         if (load_step == XS) {
             load_step = 0;
-            load_tile += gridDim.x;
+            ++load_tile;
             aim();
         }
     };
@@ -481,8 +495,10 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(con
         for (int i = 0; i < 2; ++i) {
             acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g0[i], x0[j + i], acc_g, 0, 0, 0);
             acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g1[i], x1[j + i], acc_g, 0, 0, 0);
-            acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u0[i], x0[j + i], acc_u, 0, 0, 0);
-            acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u1[i], x1[j + i], acc_u, 0, 0, 0);
+            if (GATED) {
+                acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u0[i], x0[j + i], acc_u, 0, 0, 0);
+                acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u1[i], x1[j + i], acc_u, 0, 0, 0);
+            }
         }
     };
     int half = 0;
@@ -491,25 +507,25 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(con
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             s_acc[half][wave][0][4 * c + i][r16] = acc_g[i];
-            s_acc[half][wave][1][4 * c + i][r16] = acc_u[i];
+            if (GATED) s_acc[half][wave][NT - 1][4 * c + i][r16] = acc_u[i];
         }
         acc_g = acc_u = gf32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
         if (threadIdx.x < 256) {
             const int m = threadIdx.x / 16, n = threadIdx.x % 16;
-            const int64_t col = (int64_t)tile * 16 + n;
-            if (m < M && col < rows) {
+            const int64_t col = (int64_t)tile_begin(tile) + n;
+            if (m < M && col < tile_end(tile)) {
                 float g = 0.f, u = 0.f;
 #pragma unroll
                 for (int w = 0; w < WAVES; ++w) {
                     g += s_acc[half][w][0][n][m];
-                    u += s_acc[half][w][1][n][m];
+                    if (GATED) u += s_acc[half][w][NT - 1][n][m];
                 }
                 if (SCALED) {
                     g *= s_inv[m];
                     u *= s_inv[m];
                 }
-                C[(int64_t)m * rows + col] = (bf16_t)(g / (1.0f + expf(-g)) * u);
+                C[(int64_t)m * rows + col] = (bf16_t)(GATED ? g / (1.0f + expf(-g)) * u : g);
             }
         }
         // The other half is written next; this one again only after the next tile's barrier,
@@ -517,8 +533,8 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(con
         half ^= 1;
     };
 
-    int tile = blockIdx.x;
-    for (; tile + (int)gridDim.x < tiles; tile += gridDim.x) {  // every tile of this workgroup but its last
+    int tile = 0;
+    for (; tile + 1 < tiles; ++tile) {  // every tile of the share but its last
 #pragma unroll
         for (int j = 0; j < XS; j += 4) {
             load(b);
@@ -528,16 +544,15 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_gated_stream_kernel(con
         }
         finish_tile(tile);
     }
-    if (tile < tiles) {  // the last one asks for nothing beyond itself
+    // the last one asks for nothing beyond itself
 #pragma unroll
-        for (int j = 0; j < XS; j += 4) {
-            load(b);
-            multiply(a, j);
-            if (j + 4 < XS) load(a);
-            multiply(b, j + 2);
-        }
-        finish_tile(tile);
+    for (int j = 0; j < XS; j += 4) {
+        load(b);
+        multiply(a, j);
+        if (j + 4 < XS) load(a);
+        multiply(b, j + 2);
     }
+    finish_tile(tile);
 }
 
 // CUs of the current device (asked once per device)
@@ -554,18 +569,18 @@ static int gemm_compute_units() {
 }
 
 // The streaming kernel takes the product when its shape is the one it is built for (K = 4096,
-// up to 16 rows) and every workgroup gets at least two tiles and all of them about the same
-// number (one a CU; a last round that most CUs sit out would cost more than the stream gains).
-template <bool SCALED>
-static bool launch_gated_stream(const bf16_t* X, const bf16_t* W, bf16_t* C, int M, int N, int K, const NormFold& fold,
-                                hipStream_t stream) {
+// up to 16 rows) and W has more than one tile of rows for every CU.
+template <bool GATED, bool SCALED>
+static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, bf16_t* C, int M, int N, int K,
+                                 const NormFold& fold, hipStream_t stream) {
     constexpr int XS = 4;
     if (M > 16 || K != SK_KSTEP * 16 * XS) return false;
-    const int tiles = (N / 2 + 15) / 16;
-    const int blocks = gemm_compute_units();
-    const int rounds = (tiles + blocks - 1) / blocks;
-    if (rounds < 2 || (int64_t)rounds * blocks * 9 > (int64_t)tiles * 10) return false;
-    gemm_gated_stream_kernel<SCALED, XS><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, fold);
+    const int rows = GATED ? N / 2 : N;
+    const int units = gemm_compute_units();
+    const int share = (rows + units - 1) / units;
+    if (share <= 16) return false;
+    const int blocks = (rows + share - 1) / share;
+    gemm_skinny_stream_kernel<GATED, SCALED, XS><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
     return true;
 }
 
@@ -607,7 +622,7 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
                                           hipStream_t stream) {
     if (M <= 0 || N2 <= 0) return 0;
     if (M > 32 || K % 8 != 0 || K <= 0 || N2 % 2 != 0) return (int)hipErrorInvalidValue;
-    if (launch_gated_stream<false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, NormFold{}, stream))
+    if (launch_skinny_stream<true, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, NormFold{}, stream))
         LLE_RETURN_LAUNCH_STATUS();
     return launch_skinny<bf16_t, 2, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, stream);
 }
@@ -652,7 +667,8 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     const bf16_t* w = (const bf16_t*)W;
     bf16_t* c = (bf16_t*)C;
     const int threads = 16 * LLE_WAVE;
-    if (gated && launch_gated_stream<true>(x, w, c, M, N, K, fold, stream)) {
+    if (gated && launch_skinny_stream<true, true>(x, w, c, M, N, K, fold, stream)) {
+    } else if (!gated && launch_skinny_stream<false, true>(x, w, c, M, N, K, fold, stream)) {
     } else if (gated && M <= 16)
         gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
     else if (gated)
