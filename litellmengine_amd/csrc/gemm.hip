@@ -413,10 +413,10 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 // partial tiles are added up in LDS and written out.  X is read once per workgroup
 // instead of once per tile, and the sums of the folded norm are added up once.
 // ---------------------------------------------------------------------------------
-template <bool GATED, bool SCALED, int XS>
+template <bool GATED, bool SCALED, int XS, typename TC>
 __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X,
                                                                               const bf16_t* __restrict__ W,
-                                                                              bf16_t* __restrict__ C, int M, int N, int K,
+                                                                              TC* __restrict__ C, int M, int N, int K,
                                                                               int share, NormFold fold) {
     static_assert(XS % 4 == 0, "sets of two steps of W are multiplied in pairs");
     constexpr int WAVES = 16;
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
                     g *= s_inv[m];
                     u *= s_inv[m];
                 }
-                C[(int64_t)m * rows + col] = (bf16_t)(GATED ? g / (1.0f + expf(-g)) * u : g);
+                C[(int64_t)m * rows + col] = from_f32<TC>(GATED ? g / (1.0f + expf(-g)) * u : g);
             }
         }
         // The other half is written next; this one again only after the next tile's barrier,
@@ -570,8 +570,8 @@ static int gemm_compute_units() {
 
 // The streaming kernel takes the product when its shape is the one it is built for (K = 4096,
 // up to 16 rows) and W has more than one tile of rows for every CU.
-template <bool GATED, bool SCALED>
-static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, bf16_t* C, int M, int N, int K,
+template <bool GATED, bool SCALED, typename TC>
+static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K,
                                  const NormFold& fold, hipStream_t stream) {
     constexpr int XS = 4;
     if (M > 16 || K != SK_KSTEP * 16 * XS) return false;
@@ -580,7 +580,7 @@ static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, bf16_t* C, in
     const int share = (rows + units - 1) / units;
     if (share <= 16) return false;
     const int blocks = (rows + share - 1) / share;
-    gemm_skinny_stream_kernel<GATED, SCALED, XS><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
+    gemm_skinny_stream_kernel<GATED, SCALED, XS, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
     return true;
 }
 
@@ -611,8 +611,14 @@ extern "C" int lle_gemm_skinny_bf16(const void* X, const void* W, void* C, int M
     const bf16_t* w = (const bf16_t*)W;
     // one tile of W rows per workgroup measured best up to 16 rows of X (two tiles share the X
     // operands but halve the number of workgroups; they only pay off from 16 rows on)
-    if (out_dtype == LLE_F32) return launch_skinny<float, 1, false>(x, w, (float*)C, M, N, K, stream);
-    if (out_dtype == LLE_BF16) return launch_skinny<bf16_t, 1, false>(x, w, (bf16_t*)C, M, N, K, stream);
+    if (out_dtype == LLE_F32) {
+        if (launch_skinny_stream<false, false, float>(x, w, (float*)C, M, N, K, NormFold{}, stream)) LLE_RETURN_LAUNCH_STATUS();
+        return launch_skinny<float, 1, false>(x, w, (float*)C, M, N, K, stream);
+    }
+    if (out_dtype == LLE_BF16) {
+        if (launch_skinny_stream<false, false, bf16_t>(x, w, (bf16_t*)C, M, N, K, NormFold{}, stream)) LLE_RETURN_LAUNCH_STATUS();
+        return launch_skinny<bf16_t, 1, false>(x, w, (bf16_t*)C, M, N, K, stream);
+    }
     return (int)hipErrorInvalidValue;
 }
 
@@ -622,7 +628,7 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
                                           hipStream_t stream) {
     if (M <= 0 || N2 <= 0) return 0;
     if (M > 32 || K % 8 != 0 || K <= 0 || N2 % 2 != 0) return (int)hipErrorInvalidValue;
-    if (launch_skinny_stream<true, false>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, NormFold{}, stream))
+    if (launch_skinny_stream<true, false, bf16_t>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, NormFold{}, stream))
         LLE_RETURN_LAUNCH_STATUS();
     return launch_skinny<bf16_t, 2, true>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N2, K, stream);
 }
@@ -667,8 +673,8 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     const bf16_t* w = (const bf16_t*)W;
     bf16_t* c = (bf16_t*)C;
     const int threads = 16 * LLE_WAVE;
-    if (gated && launch_skinny_stream<true, true>(x, w, c, M, N, K, fold, stream)) {
-    } else if (!gated && launch_skinny_stream<false, true>(x, w, c, M, N, K, fold, stream)) {
+    if (gated && launch_skinny_stream<true, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
+    } else if (!gated && launch_skinny_stream<false, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
     } else if (gated && M <= 16)
         gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
     else if (gated)

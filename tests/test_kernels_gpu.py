@@ -160,7 +160,7 @@ def test_silu_mul_reference_vector():
                                                 (torch.bfloat16, torch.bfloat16)])
 @pytest.mark.parametrize("M,N,K", [(1, 503, 96), (2, 4, 3), (5, 130, 70), (67, 257, 200), (33, 1000, 4096),
                                    (8, 6144, 4096), (16, 311, 136), (17, 48, 64), (64, 4096, 1536), (49, 72, 40),
-                                   (3, 151936, 128)])
+                                   (3, 151936, 128), (5, 8189, 4096), (2, 6151, 4096), (16, 4112, 4096)])
 def test_linear(in_dtype, out_dtype, M, N, K):
     x = rnd((M, K), in_dtype, 6)
     w = rnd((N, K), in_dtype, 7, 0.05)
