@@ -207,9 +207,10 @@ class HipOps:
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
 
-    # measured on MI355X: the weight-streaming kernel wins up to 8 rows for every weight, up to 16
-    # rows for weights of up to 32 Mi elements; above, the library product
-    SKINNY_MAX_ROWS = 8
+    # measured on MI355X: the weight-streaming kernels (with the norm folded into them) win up to 16
+    # rows, one tile of matrix-core columns, for every weight (batch 12 / 16 of the 8B sizes: 14 % / 10 %
+    # faster than the library products beside separate norms); up to 32 rows for small weights
+    SKINNY_MAX_ROWS = 16
     SKINNY_F32_MAX_ROWS = 64  # the float32 twin: the plain-FMA kernel it replaces wastes its 64-row tiles on few rows
     SKINNY_SMALL_WEIGHT = 1 << 25
     SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 32 rows

@@ -101,7 +101,7 @@ def test_gate_up_silu(dtype, M, I, K):
 
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M,H,K,N", [(1, 64, 40, 48), (3, 136, 72, 100), (8, 4096, 1024, 512), (5, 1000, 64, 30),
-                                     (6, 4096, 256, 8189), (1, 4096, 128, 12288),
+                                     (6, 4096, 256, 8189), (1, 4096, 128, 12288), (16, 4096, 256, 6151), (11, 5120, 128, 260),
                                      (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70), (32, 1024, 2048, 3072),
                                      (17, 72, 40, 22), (29, 2048, 512, 128)])
 def test_norm_folded_into_products(wdtype, M, H, K, N):
@@ -113,7 +113,7 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
 
     o = ops()
     assert o.can_fold_norm(M, H, torch.bfloat16) and not o.can_fold_norm(33, H, torch.bfloat16)
-    assert o.can_fold_norm(9, H, torch.bfloat16) == (H <= 2048), "more than 8 rows only for narrow models"
+    assert o.can_fold_norm(17, H, torch.bfloat16) == (H <= 2048), "more than 16 rows only for narrow models"
     assert not o.can_fold_norm(M, H, torch.float32) and not o.can_fold_norm(M, H + 4, torch.bfloat16)
     a = rnd((M, K), torch.bfloat16, 31)
     w1 = rnd((H, K), torch.bfloat16, 32, 0.2)
