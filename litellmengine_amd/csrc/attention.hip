@@ -788,7 +788,10 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 #define PRE_RT_MAX 2
 #endif
 #define PRE_RT_OF(DK) ((DK) <= 4 ? PRE_RT_MAX : 1)
-template <int DK>
+// PRE_RT row tiles per wavefront: two share every operand that is read from LDS; one gives twice the
+// workgroups of half the height, which fills the chip better when a launch is only one round of
+// them and the causal mask makes them unequal (a prompt from its first token).
+template <int DK, int PRE_RT>
 // (heads over 192 elements need more than the 256 registers a lane that two workgroups a CU leave)
 __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
@@ -797,7 +800,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     float* __restrict__ ws_ml, int ws_stride, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages,
     int window, float scale_log2, int complement_order) {
     constexpr int D = DK * 32;
-    constexpr int PRE_RT = PRE_RT_OF(DK);
+    static_assert(PRE_RT <= PRE_RT_OF(DK), "the accumulators of two row tiles fit the registers up to heads of 128");
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
     constexpr int KROW = D + 8;       // elements per key row in LDS
     constexpr int VROW = KSTEP + 8;   // elements per value-element row in LDS: 16-byte pieces stay aligned
@@ -1093,7 +1096,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
                        const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
                        int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
                        int run_decode, int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                       const FusedQKV& fused, hipStream_t stream) {
+                       int prefill_row_tiles, const FusedQKV& fused, hipStream_t stream) {
     constexpr int D = DK * 32;
     const int G = nq / nkv;
     if (!run_decode) nsplit_decode = 1;
@@ -1117,13 +1120,20 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
         if (e != 0) return e;
     }
     if (run_prefill) {
-        constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT_OF(DK);
         const int rows = max_q_len * G;
-        const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
-        const int64_t workgroups = (int64_t)nkv * blocks * nsplit_prefill * S;
-        mfma_prefill_kernel<DK><<<dim3(nkv, blocks * nsplit_prefill, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
-            q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill, nq,
-            nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0);
+        auto launch = [&](auto rt) {
+            constexpr int RT = decltype(rt)::value;
+            constexpr int PRE_ROWS = PRE_WAVES * 16 * RT;
+            const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
+            const int64_t workgroups = (int64_t)nkv * blocks * nsplit_prefill * S;
+            mfma_prefill_kernel<DK, RT><<<dim3(nkv, blocks * nsplit_prefill, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
+                q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill,
+                nq, nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0);
+        };
+        if (PRE_RT_OF(DK) == 1 || prefill_row_tiles == 1)
+            launch(std::integral_constant<int, 1>{});
+        else
+            launch(std::integral_constant<int, PRE_RT_OF(DK)>{});
     }
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
         mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(
@@ -1142,7 +1152,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d, int page_size,
                                 int64_t page_stride, int max_pages, int window, float scale, int run_decode,
                                 int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                                const FusedQKV& fused, hipStream_t stream) {
+                                int prefill_row_tiles, const FusedQKV& fused, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv > 65535) return (int)hipErrorInvalidValue;
@@ -1155,7 +1165,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
                                 (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
                                 page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit_decode,   \
-                                run_prefill, nsplit_prefill, max_q_len, fused, stream);
+                                run_prefill, nsplit_prefill, max_q_len, prefill_row_tiles, fused, stream);
     switch (d / 32) {
         LLE_ATT_CASE(1)
         LLE_ATT_CASE(2)
@@ -1175,11 +1185,12 @@ extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, con
                                         const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
                                         int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
                                         int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
-                                        int nsplit_prefill, int max_q_len, hipStream_t stream) {
+                                        int nsplit_prefill, int max_q_len, int prefill_row_tiles,
+                                        hipStream_t stream) {
     const FusedQKV none = {};
     return paged_attention_mfma(q, (void*)kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
                                 ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, run_decode,
-                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, none, stream);
+                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, prefill_row_tiles, none, stream);
 }
 
 // Decode steps only (every request has at most 16 / group tokens), head_dim a multiple of 64, a
@@ -1208,5 +1219,5 @@ extern "C" int lle_qk_norm_rope_attention_decode(const void* qkv, const void* sl
     fused.write_kv = write_kv;
     return paged_attention_mfma(nullptr, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
                                 ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, 1,
-                                nsplit_decode, 0, 1, 1, fused, stream);
+                                nsplit_decode, 0, 1, 1, 0, fused, stream);
 }
