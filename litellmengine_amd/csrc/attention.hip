@@ -734,12 +734,15 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     if (nsplit <= 1) return;
     const int lane = threadIdx.x;
     const int64_t head_row = tok * nq + h;
-    float m = NEG_BIG, l = 0.f;
-    if (lane < nsplit) {
-        const float2 ml = *(const float2*)(ws_ml + (head_row * ws_stride + lane) * 2);
-        m = ml.x;
-        l = ml.y;
-    }
+    // (m, l) of the lane's split and the first eight splits' partial sums of the lane's first two
+    // elements are asked for together: the launch is as short as its chain of loads.
+    const float* o = ws_o + head_row * ws_stride * D;
+    const float2 ml = *(const float2*)(ws_ml + (head_row * ws_stride + min(lane, nsplit - 1)) * 2);
+    const int e_first = min(2 * lane, D - 2);
+    float2 first[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) first[j] = *(const float2*)(o + (int64_t)min(j, nsplit - 1) * D + e_first);
+    const float m = lane < nsplit ? ml.x : NEG_BIG, l = lane < nsplit ? ml.y : 0.f;
     const float big = wave_max(m);
     const float f = exp2f(m - big);  // 0 for lanes without a split (l = 0 there anyway)
     const float den = wave_sum(l * f);
@@ -749,13 +752,17 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
     __syncthreads();
     // A lane takes two neighbouring elements; the partial sums of eight splits are loaded
     // together (one load after the other would pay the memory's latency once per split).
-    const float* o = ws_o + head_row * ws_stride * D;
     for (int e = 2 * lane; e < D; e += 2 * LLE_WAVE) {
         float2 num = {0.f, 0.f};
         for (int k0 = 0; k0 < nsplit; k0 += 8) {
             float2 part[8];
+            if (k0 == 0 && e == e_first) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) part[j] = *(const float2*)(o + (int64_t)min(k0 + j, nsplit - 1) * D + e);
+                for (int j = 0; j < 8; ++j) part[j] = first[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) part[j] = *(const float2*)(o + (int64_t)min(k0 + j, nsplit - 1) * D + e);
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float fk = k0 + j < nsplit ? s_f[k0 + j] : 0.f;
