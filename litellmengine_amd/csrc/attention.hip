@@ -35,6 +35,7 @@ LLE_DEFINE_ERROR_STRING()
 
 #define ATT_WAVES 4
 #define ATT_MAX_R 4  // head_dim <= 256
+#define ATT_KEYS 4   // keys a wavefront works on at a time
 
 template <typename T>
 __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_kernel(
@@ -66,27 +67,79 @@ __global__ __launch_bounds__(ATT_WAVES* LLE_WAVE) void paged_attention_generic_k
     }
     float m = -FLT_MAX, l = 0.f;
     const int64_t v_base = ((int64_t)nkv + kvh) * page_size * d;
-    for (int j = lo + wave; j <= pos; j += ATT_WAVES) {
-        const int lp = j / page_size;
-        const int off = j - lp * page_size;
-        const T* page = kv_layer + (int64_t)table[lp] * page_stride;
-        const T* kp = page + ((int64_t)kvh * page_size + off) * d;
-        const T* vp = page + v_base + off;  // element e of the value row at vp[e * page_size]
-        float dot = 0.f;
+    // A wavefront takes ATT_KEYS consecutive keys at a time, so that the loads of several keys
+    // are on their way together (one key after the other, each would wait for its own K row and
+    // then for its own V row).  Which keys share a step depends on (lo, pos) only.
+    // (keys j0 .. j0 + ATT_KEYS - 1 lie in one page, side by side, when the steps start at a
+    // multiple of ATT_KEYS and pages hold a multiple of it; the last step of a row may reach
+    // past `pos`, but not past its page)
+    const bool keys_in_one_piece = lo % ATT_KEYS == 0 && page_size % ATT_KEYS == 0;
+    for (int j0 = lo + wave * ATT_KEYS; j0 <= pos; j0 += ATT_WAVES * ATT_KEYS) {
+        const T* vp[ATT_KEYS];
+        float dot[ATT_KEYS];
 #pragma unroll
-        for (int r = 0; r < ATT_MAX_R; ++r) {
-            const int e = lane + LLE_WAVE * r;
-            if (e < d) dot += qv[r] * to_f32<T>(kp[e]);
+        for (int i = 0; i < ATT_KEYS; ++i) {
+            const int j = min(j0 + i, pos);  // past the row's last key: that key again, weighted 0 below
+            const int lp = j / page_size;
+            const int off = j - lp * page_size;
+            // the same for the whole wavefront: a scalar load
+            const T* page = kv_layer + (int64_t)table[__builtin_amdgcn_readfirstlane(lp)] * page_stride;
+            const T* kp = page + ((int64_t)kvh * page_size + off) * d;
+            vp[i] = page + v_base + off;  // element e of the value row at vp[e * page_size]
+            dot[i] = 0.f;
+#pragma unroll
+            for (int r = 0; r < ATT_MAX_R; ++r) {
+                const int e = lane + LLE_WAVE * r;
+                if (e < d) dot[i] += qv[r] * to_f32<T>(kp[e]);
+            }
         }
-        const float score = wave_sum(dot) * scale;
-        const float new_m = fmaxf(m, score);
+        float vals[ATT_KEYS][ATT_MAX_R];
+        if (keys_in_one_piece) {
+            // the ATT_KEYS values of an element lie side by side in the page: one load for all of them
+            typedef T piece_t __attribute__((ext_vector_type(ATT_KEYS)));
+#pragma unroll
+            for (int r = 0; r < ATT_MAX_R; ++r) {
+                const int e = lane + LLE_WAVE * r;
+                if (e < d) {
+                    const piece_t piece = *(const piece_t*)(vp[0] + (int64_t)e * page_size);
+#pragma unroll
+                    for (int i = 0; i < ATT_KEYS; ++i)  // what lies past `pos` was never written: not even times 0
+                        vals[i][r] = j0 + i <= pos ? to_f32<T>(piece[i]) : 0.f;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < ATT_KEYS; ++i) vals[i][r] = 0.f;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < ATT_KEYS; ++i)
+#pragma unroll
+                for (int r = 0; r < ATT_MAX_R; ++r) {
+                    const int e = lane + LLE_WAVE * r;
+                    vals[i][r] = e < d ? to_f32<T>(vp[i][(int64_t)e * page_size]) : 0.f;
+                }
+        }
+        float score[ATT_KEYS];
+        float new_m = m;
+#pragma unroll
+        for (int i = 0; i < ATT_KEYS; ++i) {
+            score[i] = wave_sum(dot[i]) * scale;
+            if (j0 + i <= pos) new_m = fmaxf(new_m, score[i]);
+        }
         const float alpha = expf(m - new_m);
-        const float beta = expf(score - new_m);
-        l = l * alpha + beta;
+        float beta[ATT_KEYS];
+        l *= alpha;
+#pragma unroll
+        for (int i = 0; i < ATT_KEYS; ++i) {
+            beta[i] = j0 + i <= pos ? expf(score[i] - new_m) : 0.f;
+            l += beta[i];
+        }
 #pragma unroll
         for (int r = 0; r < ATT_MAX_R; ++r) {
-            const int e = lane + LLE_WAVE * r;
-            if (e < d) acc[r] = acc[r] * alpha + beta * to_f32<T>(vp[(int64_t)e * page_size]);
+            float a = acc[r] * alpha;
+#pragma unroll
+            for (int i = 0; i < ATT_KEYS; ++i) a += beta[i] * vals[i][r];
+            acc[r] = a;
         }
         m = new_m;
     }
