@@ -374,6 +374,7 @@ class HipOps:
         return out
 
     force_generic_attention = False  # tests flip this to compare the two families of kernels
+    force_prefill_row_tiles = 0      # tests set 1 or 2 to reach both heights of the prompt-portion workgroups
     force_separate_rope = False      # tests flip this to compare the fused decode step with its two halves
     # measured on MI355X: about one workgroup per CU and at least 8 32-key steps (two per
     # wavefront) per split are best; more splits cost more in partial results than they gain
@@ -406,6 +407,8 @@ class HipOps:
         portion or more the taller workgroups win by 20-30 %."""
         if head_dim > 128:
             return 1
+        if self.force_prefill_row_tiles:
+            return self.force_prefill_row_tiles
         key = device.index if device.index is not None else torch.cuda.current_device()
         if key not in self._compute_units:
             self._compute_units[key] = torch.cuda.get_device_properties(key).multi_processor_count
