@@ -19,17 +19,43 @@ Pool layout of a group: [layer, page, 2 (K, V), kv_head, page_size, head_dim].
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
+from array import array
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
 from ..parts.base import KVCacheSpec, StateSpec
-from .page_pool import OutOfPages, PagePool
+from .page_pool import OK, TOO_MANY_PAGES, OutOfPages, PagePool, PageTables
+
+
+class _TableView:
+    """`group.tables[slot]`: a request slot's block table as a list (a copy of the native one)."""
+
+    def __init__(self, group: "CacheGroup"):
+        self._group = group
+
+    def __len__(self) -> int:
+        return self._group.max_requests
+
+    def __getitem__(self, slot: int) -> List[int]:
+        g = self._group
+        if not 0 <= slot < g.max_requests:
+            raise IndexError(slot)
+        n = g._lib.lle_pt_table_len(g._h, slot)
+        out = (ctypes.c_int32 * max(1, n))()
+        g._lib.lle_pt_table_copy(g._h, slot, out)
+        return list(out[:n])
+
+    def __iter__(self):
+        return (self[slot] for slot in range(len(self)))
 
 
 class CacheGroup:
-    """Pages, pool and block tables of the cache layers that share one KVCacheSpec."""
+    """Pages, pool and block tables of the cache layers that share one KVCacheSpec.  The
+    bookkeeping (free list, tables, what has not reached the device table yet) is the native
+    host library's; the pool and the device table are tensors held here."""
 
     def __init__(self, index: int, spec: KVCacheSpec, cache_ids: Sequence[int], page_size: int, num_pages: int,
                  max_requests: int, max_pages_per_request: int, dtype: torch.dtype, device: torch.device):
@@ -38,64 +64,63 @@ class CacheGroup:
         self.cache_ids = list(cache_ids)
         self.page_size = page_size
         self.window = spec.window
-        self.pool = PagePool(num_pages)
+        self.max_requests = max_requests
         self.max_pages_per_request = max_pages_per_request
+        self.native = PageTables(num_pages, page_size, max_requests, max_pages_per_request, spec.window)
+        self._lib, self._h = self.native.lib, self.native.handle
+        self.pool = PagePool(num_pages, self.native)
         self.kv = torch.zeros(
             (len(self.cache_ids), num_pages, 2, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype, device=device
         )
         # per request slot: logical page -> physical page (-1 once the window has passed it)
-        self.tables: List[List[int]] = [[] for _ in range(max_requests)]
-        self.first_live: List[int] = [0] * max_requests
+        self.tables = _TableView(self)
         self.block_table = torch.full((max_requests, max_pages_per_request), -1, dtype=torch.int32, device=device)
-        self.pending: Dict[int, int] = {}  # flat index into block_table -> page, not yet on the device
         self.slot_mapping: Optional[torch.Tensor] = None  # int32 [N] of the step being run
 
     def pages_for(self, length: int) -> int:
         return (length + self.page_size - 1) // self.page_size
 
+    def table_len(self, slot: int) -> int:
+        return self._lib.lle_pt_table_len(self._h, slot)
+
     def new_pages_needed(self, slot: int, new_len: int) -> int:
-        return max(0, self.pages_for(new_len) - len(self.tables[slot]))
+        return self._lib.lle_pt_new_pages_needed(self._h, slot, new_len)
 
     def grow(self, slot: int, new_len: int) -> None:
-        need = self.new_pages_needed(slot, new_len)
-        if need == 0:
-            return
-        table = self.tables[slot]
-        if len(table) + need > self.max_pages_per_request:
+        code = self._lib.lle_pt_grow(self._h, slot, new_len)
+        if code == TOO_MANY_PAGES:
             raise OutOfPages(
                 f"a request may hold {self.max_pages_per_request} pages of {self.page_size} tokens; "
-                f"{new_len} tokens need {len(table) + need}"
+                f"{new_len} tokens need {self.pages_for(new_len)}"
             )
-        for page in self.pool.allocate(need):
-            self.pending[slot * self.max_pages_per_request + len(table)] = page
-            table.append(page)
+        if code != OK:
+            raise OutOfPages(f"not enough free physical blocks: {self.pool.num_free} free")
 
     def trim(self, slot: int, length: int) -> None:
         """Give back the pages that no later query can see: with a window w the
         next query (position `length`) sees keys >= length - w + 1."""
-        if self.window is None:
-            return
-        first_needed = max(0, length - self.window + 1) // self.page_size
-        table = self.tables[slot]
-        first = self.first_live[slot]
-        if first_needed > first:
-            last = min(first_needed, len(table))
-            self.pool.release([table[i] for i in range(first, last)])
-            for i in range(first, last):
-                table[i] = -1
-            self.first_live[slot] = last
+        self._lib.lle_pt_trim(self._h, slot, length)
 
     def release(self, slot: int) -> None:
-        table = self.tables[slot]
-        self.pool.release([p for p in table[self.first_live[slot]:]])
-        self.tables[slot] = []
-        self.first_live[slot] = 0
+        self._lib.lle_pt_release_slot(self._h, slot)
 
     def token_slot(self, slot: int, pos: int) -> int:
-        page = self.tables[slot][pos // self.page_size]
-        if page < 0:
+        where = self._lib.lle_pt_token_slot(self._h, slot, pos)
+        if where == -2:
             raise IndexError(f"position {pos} lies in a page that was given back")
-        return page * self.page_size + pos % self.page_size
+        if where < 0:
+            raise IndexError(f"position {pos} has no page")
+        return where
+
+    def take_pending(self) -> Tuple[List[int], List[int]]:
+        """(flat indices into the device table, pages) of entries made since the last call."""
+        n = self._lib.lle_pt_num_pending(self._h)
+        if n == 0:
+            return [], []
+        index, pages = (ctypes.c_int32 * n)(), (ctypes.c_int32 * n)()
+        self._lib.lle_pt_take_pending(self._h, index, pages)
+        latest = dict(zip(index, pages))  # an entry made twice (a slot given back and used again): the later one
+        return list(latest.keys()), list(latest.values())
 
     def apply_table_updates(self, flat_index: torch.Tensor, pages: torch.Tensor) -> None:
         """Write new table entries (int32 device arrays) into the device table."""
@@ -199,18 +224,22 @@ class CacheManager:
             raise ValueError(f"request slot {slot} is not in use")
 
     # -- pages -----------------------------------------------------------------------
-    def can_extend(self, wants: Sequence[Tuple[int, int]]) -> bool:
-        """Would `extend_many(wants)` succeed?  wants = [(slot, new_len), ...]."""
+    @staticmethod
+    def _arrays(wants: Sequence[Tuple[int, int]]):
+        slots, lens = array("i", (w[0] for w in wants)), array("i", (w[1] for w in wants))
+        return len(wants), slots.buffer_info()[0], lens.buffer_info()[0], (slots, lens)
+
+    def _can_extend(self, n: int, slots: int, lens: int) -> bool:
         for group in self.groups:
-            need = 0
-            for slot, new_len in wants:
-                n = group.new_pages_needed(slot, new_len)
-                if len(group.tables[slot]) + n > group.max_pages_per_request:
-                    return False
-                need += n
-            if need > group.pool.num_free:
+            need = group._lib.lle_pt_pages_needed_many(group._h, n, slots, lens)
+            if need < 0 or need > group.pool.num_free:
                 return False
         return True
+
+    def can_extend(self, wants: Sequence[Tuple[int, int]]) -> bool:
+        """Would `extend_many(wants)` succeed?  wants = [(slot, new_len), ...]."""
+        n, slots, lens, keep = self._arrays(wants)
+        return self._can_extend(n, slots, lens)
 
     def extend_many(self, wants: Sequence[Tuple[int, int]]) -> None:
         """Make room for positions < new_len of every (slot, new_len): all or nothing."""
@@ -218,12 +247,13 @@ class CacheManager:
             self._check_live(slot)
             if new_len < self._length[slot]:
                 raise ValueError("a request cannot shrink")
-        if not self.can_extend(wants):
+        n, slots, lens, keep = self._arrays(wants)
+        if not self._can_extend(n, slots, lens):
             free = ", ".join(f"group {g.index}: {g.pool.num_free}" for g in self.groups)
             raise OutOfPages(f"not enough free physical blocks for this step (free pages: {free})")
         for group in self.groups:
-            for slot, new_len in wants:
-                group.grow(slot, new_len)
+            if group._lib.lle_pt_grow_many(group._h, n, slots, lens) != OK:
+                raise RuntimeError("the pages of a group changed between the check and the growth")
 
     def extend(self, slot: int, new_len: int) -> None:
         self.extend_many([(slot, new_len)])
@@ -233,7 +263,18 @@ class CacheManager:
         self._check_live(slot)
         self._length[slot] = new_len
         for group in self.groups:
-            group.trim(slot, new_len)
+            if group.window is not None:
+                group.trim(slot, new_len)
+
+    def commit_many(self, wants: Sequence[Tuple[int, int]]) -> None:
+        """commit() for every (slot, new_len) of a step."""
+        for slot, new_len in wants:
+            self._check_live(slot)
+            self._length[slot] = new_len
+        if any(group.window is not None for group in self.groups):
+            n, slots, lens, keep = self._arrays(wants)
+            for group in self.groups:
+                group._lib.lle_pt_trim_many(group._h, n, slots, lens)
 
     def free_pages(self) -> List[int]:
         return [g.pool.num_free for g in self.groups]
@@ -252,7 +293,7 @@ class CacheManager:
         """[(group index, flat indices, pages)] of table entries not yet on the device."""
         out = []
         for g in self.groups:
-            if g.pending:
-                out.append((g.index, list(g.pending.keys()), list(g.pending.values())))
-                g.pending = {}
+            index, pages = g.take_pending()
+            if index:
+                out.append((g.index, index, pages))
         return out

@@ -1,4 +1,6 @@
-"""Builds and loads the HIP libraries of this package (gfx950 only).
+"""Builds and loads the native libraries of this package: the HIP kernels (gfx950
+only) and the host-side bookkeeping of the cache and of a step (`host.cpp`, C++
+without GPU code, compiled with the host compiler).
 
 Every `.hip` file here becomes one shared library, compiled with hipcc the
 first time something needs it and loaded with ctypes.  A library is rebuilt
@@ -31,6 +33,9 @@ LIBRARIES: Dict[str, List[str]] = {
     "gemm": ["gemm.hip"],
     "sampling": ["sampling.hip"],
 }
+# libraries without GPU code: compiled with the host's C++ compiler
+HOST_LIBRARIES: Dict[str, List[str]] = {"host": ["host.cpp"]}
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
 HEADERS = ["common.h"]
 # packed 32-bit float instructions are switched off on purpose (device flag)
 FLAGS = [
@@ -94,10 +99,19 @@ def lib_dir() -> str:
         return _lib_dir
 
 
+def _host_compiler() -> str:
+    for cand in ("g++", "c++", "clang++"):
+        exe = shutil.which(cand)
+        if exe:
+            return exe
+    return _hipcc()  # compiles plain C++ as well
+
+
 def _source_hash(name: str) -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
-    for fn in HEADERS + LIBRARIES[name]:
+    host = name in HOST_LIBRARIES
+    h.update(" ".join(HOST_FLAGS if host else FLAGS).encode())
+    for fn in (HOST_LIBRARIES[name] if host else HEADERS + LIBRARIES[name]):
         with open(os.path.join(_HERE, fn), "rb") as f:
             h.update(fn.encode())
             h.update(f.read())
@@ -125,14 +139,19 @@ def _find_built(name: str):
 
 def compile_library(name: str, verbose: bool = True) -> str:
     """Compile one library now (whether or not a built one exists)."""
-    if name not in LIBRARIES:
-        raise BuildError(f"unknown kernel library {name!r}")
+    if name not in LIBRARIES and name not in HOST_LIBRARIES:
+        raise BuildError(f"unknown library {name!r}")
     directory = lib_dir()
     so, hs = _paths(name, directory)
     tmp = f"{so}.{os.getpid()}.{threading.get_ident()}.tmp"
-    cmd = [_hipcc()] + FLAGS + [os.path.join(_HERE, s) for s in LIBRARIES[name]] + ["-o", tmp]
+    if name in HOST_LIBRARIES:
+        cmd = [_host_compiler()] + HOST_FLAGS + [os.path.join(_HERE, s) for s in HOST_LIBRARIES[name]] + ["-o", tmp]
+        what = f"host library '{name}'"
+    else:
+        cmd = [_hipcc()] + FLAGS + [os.path.join(_HERE, s) for s in LIBRARIES[name]] + ["-o", tmp]
+        what = f"kernels '{name}' for {ARCH}"
     if verbose:
-        print(f"[litellmengine_amd] compiling kernels '{name}' for {ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[litellmengine_amd] compiling {what} ...", file=sys.stderr, flush=True)
     t0 = time.time()
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())
@@ -158,7 +177,7 @@ def compile_library(name: str, verbose: bool = True) -> str:
             os.unlink(tmp)
         except OSError:
             pass
-        raise BuildError(f"hipcc failed for '{name}':\n{output}")
+        raise BuildError(f"{cmd[0]} failed for '{name}':\n{output}")
     os.replace(tmp, so)
     with open(hs + ".tmp", "w") as f:
         f.write(_source_hash(name))
@@ -170,7 +189,7 @@ def compile_library(name: str, verbose: bool = True) -> str:
 
 def build_all(verbose: bool = True, jobs: int = 4) -> None:
     """Compile every library, in parallel; always compiles."""
-    names = list(LIBRARIES)
+    names = list(LIBRARIES) + list(HOST_LIBRARIES)
     errors: List[BaseException] = []
     sem = threading.Semaphore(jobs)
 

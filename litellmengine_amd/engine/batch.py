@@ -9,10 +9,14 @@ device in ONE copy and are views of that buffer.
 """
 from __future__ import annotations
 
+import ctypes
 import dataclasses
+from array import array
 from typing import List, Optional, Sequence, Tuple
 
 import torch
+
+from ..cache.page_pool import BAD_TOKEN, NO_PAGE_AT_POSITION, host_library
 
 
 @dataclasses.dataclass(frozen=True)
@@ -53,9 +57,9 @@ class StepState:
 
 @dataclasses.dataclass
 class StepLayout:
-    """The host side of a step: one flat int32 list and where its parts lie."""
+    """The host side of a step: one flat int32 tensor and where its parts lie."""
 
-    flat: List[int]
+    host: torch.Tensor  # int32, on the host (pinned when the step runs on a GPU)
     num_tokens: int
     num_seqs: int
     num_logit_rows: int
@@ -68,40 +72,64 @@ class StepLayout:
         return [N, N, N, S, S + 1, S, R] + [N] * self.num_groups
 
 
-def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False) -> StepLayout:
+class _Staging:
+    """Host buffers that the native layout writes into: pinned (page-locked) when a GPU will
+    read them, grown as needed and used again by the next step (the copy to the device has
+    ended when a step's arrays are used again)."""
+
+    def __init__(self):
+        self.buffers = {}
+
+    def get(self, n: int, pinned: bool) -> torch.Tensor:
+        buf = self.buffers.get(pinned)
+        if buf is None or buf.numel() < n:
+            size = max(1024, 1 << (max(1, n) - 1).bit_length())
+            buf = torch.empty(size, dtype=torch.int32, pin_memory=pinned)
+            self.buffers[pinned] = buf
+        return buf[:n]
+
+
+_staging = _Staging()
+
+
+def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, vocab_size: int = 0,
+                device=None) -> StepLayout:
     """Lay the entries out flat and compute every token's page slot in every cache
-    group.  Pages for the new lengths must already be there.  `all_rows` asks for
-    the logits of every row whatever the entries want."""
-    token_ids: List[int] = []
-    positions: List[int] = []
-    token_seq: List[int] = []
-    seq_slots: List[int] = []
-    cu_tokens: List[int] = [0]
-    kv_lens: List[int] = []
-    logit_rows: List[int] = []
+    group (csrc/host.cpp does both).  Pages for the new lengths must already be there.
+    `all_rows` asks for the logits of every row whatever the entries want; with
+    `vocab_size` token ids outside [0, vocab_size) are refused."""
+    S = len(entries)
+    slots = array("i", (e.slot for e in entries))
+    past = array("i", (cache.length(e.slot) for e in entries))
+    q_len = array("i", (len(e.tokens) for e in entries))
+    tokens = array("i")
+    rows = array("i")
     seqs: List[SeqInfo] = []
-    for s, e in enumerate(entries):
-        past = cache.length(e.slot)
-        n = len(e.tokens)
-        start = len(token_ids)
-        token_ids.extend(int(t) for t in e.tokens)
-        positions.extend(range(past, past + n))
-        token_seq.extend([s] * n)
-        seq_slots.append(e.slot)
-        cu_tokens.append(start + n)
-        kv_lens.append(past + n)
+    start = 0
+    for e, p, n in zip(entries, past, q_len):
+        tokens.extend(e.tokens if isinstance(e.tokens, (list, array)) else [int(t) for t in e.tokens])
         if all_rows:
-            logit_rows.extend(range(start, start + n))
+            rows.extend(range(start, start + n))
         else:
-            logit_rows.extend(start + int(w) for w in e.want)
-        seqs.append(SeqInfo(e.slot, start, n, past))
-    flat: List[int] = token_ids + positions + token_seq + seq_slots + cu_tokens + kv_lens + logit_rows
-    for group in cache.groups:
-        P = group.page_size
-        for q in seqs:
-            table = group.tables[q.slot]
-            flat.extend(table[pos // P] * P + pos % P for pos in range(q.past_len, q.past_len + q.q_len))
-    return StepLayout(flat, len(token_ids), len(seqs), len(logit_rows), len(cache.groups), seqs, max(kv_lens))
+            rows.extend(start + int(w) for w in e.want)
+        seqs.append(SeqInfo(e.slot, start, n, p))
+        start += n
+    N, R, G = start, len(rows), len(cache.groups)
+    pinned = device is not None and torch.device(device).type == "cuda"
+    host = _staging.get(3 * N + 3 * S + 1 + R + G * N, pinned)
+    lib = host_library()
+    handles = (ctypes.c_void_p * max(1, G))(*[g.native.handle for g in cache.groups])
+    info = ctypes.c_int64(0)
+    address = lambda a: a.buffer_info()[0]
+    code = lib.lle_layout_step(S, address(slots), address(past), address(q_len), address(tokens), int(vocab_size), R,
+                               address(rows), G, handles, host.data_ptr(), ctypes.byref(info))
+    if code == BAD_TOKEN:
+        raise ValueError(f"token id {tokens[info.value]} outside [0, {vocab_size})")
+    if code == NO_PAGE_AT_POSITION:
+        raise IndexError(f"position {info.value} has no page: the cache was not extended for this step")
+    if code != 0:
+        raise ValueError(f"the step cannot be laid out: {lib.lle_error_string(code).decode()} (at {info.value})")
+    return StepLayout(host, N, S, R, G, seqs, max(p + n for p, n in zip(past, q_len)))
 
 
 def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:
@@ -121,7 +149,7 @@ def apply_table_updates(cache, device) -> None:
     for _, idx, pages in updates:
         flat += idx
         flat += pages
-    buf = torch.tensor(flat, dtype=torch.int32).to(device)
+    buf = torch.tensor(flat, dtype=torch.int32).to(device)  # a few entries a step
     off = 0
     for g, idx, pages in updates:
         n = len(idx)
@@ -144,9 +172,9 @@ def state_on(buf: torch.Tensor, layout: StepLayout, cache, max_kv_len: Optional[
     )
 
 
-def build_step(entries: Sequence[StepEntry], cache, device) -> StepState:
+def build_step(entries: Sequence[StepEntry], cache, device, vocab_size: int = 0) -> StepState:
     """Layout, one upload, views; also sends new block-table entries."""
-    layout = layout_step(entries, cache)
+    layout = layout_step(entries, cache, vocab_size=vocab_size, device=device)
     apply_table_updates(cache, device)
-    buf = torch.tensor(layout.flat, dtype=torch.int32).to(device)
+    buf = layout.host.to(device) if torch.device(device).type != "cpu" else layout.host.clone()
     return state_on(buf, layout, cache)

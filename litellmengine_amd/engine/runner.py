@@ -69,12 +69,17 @@ class ModelRunner:
                 raise ValueError(f"request slot {e.slot} is not in use")
             if len(e.tokens) == 0:
                 raise ValueError("an entry needs at least one token")
-            for t in e.tokens:
-                if not 0 <= int(t) < self.vocab_size:
-                    raise ValueError(f"token id {t} outside [0, {self.vocab_size})")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"wanted place {w} outside the entry's {len(e.tokens)} tokens")
+
+    def check_tokens(self, entries: Sequence[StepEntry]) -> None:
+        """Token ids outside the vocabulary are refused before anything is changed
+        (src/layers/embedding.cu:75-87).  min and max run in C."""
+        for e in entries:
+            if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size:
+                bad = next(t for t in e.tokens if not 0 <= int(t) < self.vocab_size)
+                raise ValueError(f"token id {bad} outside [0, {self.vocab_size})")
 
     def step(self, entries: Sequence[StepEntry], borrow: bool = False) -> torch.Tensor:
         """Run the entries as one batch.  Returns float32 logits [wanted, vocab] in
@@ -84,26 +89,26 @@ class ModelRunner:
         self.check(entries)
         cache = self.cache
         wants = [(e.slot, cache.length(e.slot) + len(e.tokens)) for e in entries]
+        self.check_tokens(entries)
         cache.extend_many(wants)
         if self.use_graphs and len(entries) <= self.MAX_GRAPH_BATCH and all(len(e.tokens) == 1 for e in entries):
             logits = self._graph_step(entries, borrow)
         else:
-            state = build_step(entries, cache, self.device)
+            state = build_step(entries, cache, self.device, self.vocab_size)
             self.last_step = state
             logits = self.model.forward(state, cache)
-        for slot, new_len in wants:
-            cache.commit(slot, new_len)
+        cache.commit_many(wants)
         return logits
 
     # decoding through a captured graph ---------------------------------------------------
     def _graph_step(self, entries: Sequence[StepEntry], borrow: bool) -> torch.Tensor:
         cache = self.cache
-        layout = layout_step(entries, cache, all_rows=True)
+        layout = layout_step(entries, cache, all_rows=True, vocab_size=self.vocab_size, device=self.device)
         apply_table_updates(cache, self.device)
         bucket = self.MIN_CONTEXT_BUCKET
         while bucket < layout.max_kv_len:
             bucket *= 2
-        host = torch.tensor(layout.flat, dtype=torch.int32)
+        host = layout.host
         key = (layout.num_seqs, bucket)
         g = self._graphs.get(key)
         if g is None:

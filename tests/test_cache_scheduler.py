@@ -291,3 +291,46 @@ def test_no_admission_in_a_step_that_preempted():
             s.cache.commit(p.request.slot, p.start + p.num_tokens)
         s.update(plan, [7 for p in plan if p.samples])
     assert seen_preempt
+
+
+# -- the step layout (csrc/host.cpp) ------------------------------------------------------
+def test_step_layout_matches_the_address_map():
+    """Token ids, positions, requests, lengths, wanted rows and every token's page slot in
+    every group, as one flat array: against the same computed here from the tables."""
+    from litellmengine_amd.engine.batch import StepEntry, layout_step
+
+    m = manager("C", page_size=4, num_pages=16, max_requests=4)  # two groups: a window and all keys
+    a, b, c = m.admit(), m.admit(), m.admit()
+    m.extend(a, 7)
+    m.commit(a, 7)
+    m.extend(b, 30)
+    m.commit(b, 30)  # the window group has given pages of b back
+    entries = [StepEntry(b, [9, 8, 7], [2]), StepEntry(a, [1], []), StepEntry(c, [4, 5, 6, 7, 8], [0, 4])]
+    m.extend_many([(b, 33), (a, 8), (c, 5)])
+    lay = layout_step(entries, m, vocab_size=10)
+    N, S, R, G = 9, 3, 3, len(m.groups)
+    assert (lay.num_tokens, lay.num_seqs, lay.num_logit_rows, lay.num_groups, lay.max_kv_len) == (N, S, R, G, 33)
+    flat = lay.host.tolist()
+    assert len(flat) == 3 * N + 3 * S + 1 + R + G * N
+    want = [9, 8, 7, 1, 4, 5, 6, 7, 8] + [30, 31, 32, 7, 0, 1, 2, 3, 4] + [0, 0, 0, 1, 2, 2, 2, 2, 2]
+    want += [b, a, c] + [0, 3, 4, 9] + [33, 8, 5] + [2, 4, 8]
+    for g in m.groups:
+        want += [g.token_slot(s, p) for s, p in [(b, 30), (b, 31), (b, 32), (a, 7)] + [(c, i) for i in range(5)]]
+    assert flat == want
+    assert [(q.slot, q.q_start, q.q_len, q.past_len) for q in lay.seqs] == [(b, 0, 3, 30), (a, 3, 1, 7), (c, 4, 5, 0)]
+    every = layout_step(entries, m, all_rows=True)
+    assert every.host.tolist()[3 * N + 3 * S + 1:3 * N + 3 * S + 1 + N] == list(range(N))
+
+
+def test_step_layout_refuses_bad_tokens_and_missing_pages():
+    from litellmengine_amd.engine.batch import StepEntry, layout_step
+
+    m = manager(page_size=4, num_pages=8)
+    a = m.admit()
+    m.extend(a, 4)
+    with pytest.raises(ValueError, match="token id 300 outside"):
+        layout_step([StepEntry(a, [1, 300], [])], m, vocab_size=256)
+    with pytest.raises(ValueError, match="token id -1 outside"):
+        layout_step([StepEntry(a, [-1], [])], m, vocab_size=256)
+    with pytest.raises(IndexError, match="has no page"):
+        layout_step([StepEntry(a, [1, 2, 3, 4, 5], [])], m, vocab_size=256)  # the fifth position was never extended to
