@@ -37,6 +37,8 @@ LIBRARIES: Dict[str, List[str]] = {
 HOST_LIBRARIES: Dict[str, List[str]] = {"host": ["host.cpp"]}
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared"]
 HEADERS = ["common.h"]
+# headers that only one library includes
+OWN_HEADERS: Dict[str, List[str]] = {"sampling": ["sampling.h"]}
 # packed 32-bit float instructions are switched off on purpose (device flag)
 FLAGS = [
     f"--offload-arch={ARCH}",
@@ -111,7 +113,7 @@ def _source_hash(name: str) -> str:
     h = hashlib.sha256()
     host = name in HOST_LIBRARIES
     h.update(" ".join(HOST_FLAGS if host else FLAGS).encode())
-    for fn in (HOST_LIBRARIES[name] if host else HEADERS + LIBRARIES[name]):
+    for fn in (HOST_LIBRARIES[name] if host else HEADERS + OWN_HEADERS.get(name, []) + LIBRARIES[name]):
         with open(os.path.join(_HERE, fn), "rb") as f:
             h.update(fn.encode())
             h.update(f.read())

@@ -2,8 +2,14 @@
 // argmax_each_row_kernel, src/ops/argmax.cu:181-241) and temperature sampling
 // (the reference parses --temperature and then only warns, src/main.cpp:175-178).
 #include "common.h"
+#include "sampling.h"
+#include <mutex>
 
-LLE_DEFINE_ERROR_STRING()
+extern "C" const char* lle_error_string(int code) {
+    if (code == LLE_ERROR_STATIC_SCRATCH_TOO_SMALL)
+        return "lle_argmax_rows_static takes at most 256 rows (LLE_ARGMAX_STATIC_MAX_ROWS): its buffer has a fixed size";
+    return hipGetErrorString((hipError_t)code);
+}
 
 #define SAMPLE_THREADS 1024
 
@@ -91,6 +97,52 @@ extern "C" int lle_argmax_rows(const void* logits, void* out, void* part_val, vo
                                                                           (int32_t*)part_idx, V);
     argmax_final_kernel<<<R, LLE_WAVE, 0, stream>>>((const float*)part_val, (const int32_t*)part_idx, (int32_t*)out,
                                                      chunks);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// Chunks of a row: enough workgroups to stream a long row from all CUs.
+static int argmax_chunks_for(int V) {
+    const int c = V / 2048;
+    return c < 1 ? 1 : (c > LLE_ARGMAX_STATIC_MAX_CHUNKS ? LLE_ARGMAX_STATIC_MAX_CHUNKS : c);
+}
+
+// The chunk winners of lle_argmax_rows_static: values (float) of up to MAX_ROWS * MAX_CHUNKS
+// chunks, then their indices (int32).  In host code this name is only a handle for
+// hipGetSymbolAddress; the address that kernels get is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[LLE_ARGMAX_STATIC_BYTES];
+
+static int static_scratch_address(void** ptr) {
+    static std::mutex lock;
+    static void* address[64] = {nullptr};  // per device: every GPU holds its own copy of the array
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (address[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        address[dev] = p;
+    }
+    *ptr = address[dev];
+    return 0;
+}
+
+// see sampling.h
+extern "C" int lle_argmax_rows_static(const void* logits, void* out, int R, int V, hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (V <= 0 || logits == nullptr || out == nullptr) return (int)hipErrorInvalidValue;
+    if (R > LLE_ARGMAX_STATIC_MAX_ROWS) return LLE_ERROR_STATIC_SCRATCH_TOO_SMALL;
+    void* base = nullptr;
+    const int err = static_scratch_address(&base);
+    if (err != 0) return err;
+    const int chunks = argmax_chunks_for(V);
+    float* part_val = (float*)base;
+    int32_t* part_idx = (int32_t*)((unsigned char*)base + LLE_ARGMAX_STATIC_BYTES / 2);
+    argmax_chunks_kernel<<<dim3(R, chunks), ARGMAX_THREADS, 0, stream>>>((const float*)logits, part_val, part_idx, V);
+    argmax_final_kernel<<<R, LLE_WAVE, 0, stream>>>(part_val, part_idx, (int32_t*)out, chunks);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
