@@ -146,72 +146,166 @@ extern "C" int lle_argmax_rows_static(const void* logits, void* out, int R, int 
     LLE_RETURN_LAUNCH_STATUS();
 }
 
-// p_i = exp((x_i - max) / T); the pick is the first i whose running sum of p
-// exceeds u * sum(p).  Thread t owns the contiguous ids [t c, (t + 1) c), so the
-// running sum is taken in id order.  Rows with T <= 0 are picked greedily.
+// p_i = exp((x_i - max) / T); the pick is the first i whose running sum of p exceeds
+// u * sum(p); if rounding leaves none, the last i with p_i > 0.  Rows with T <= 0 are picked
+// greedily (first maximum).  One workgroup per row, every read of the row coalesced:
+//   1. the first maximum (threads stride over the row);
+//   2. the row is cut into segments of whole 1024-element lines (one line a segment up to
+//      2 M ids); a wavefront sums a line with 16 loads of 64 neighbouring ids;
+//   3. one wavefront scans the segment sums in id order and finds the segment that the
+//      target falls into;
+//   4. the workgroup scans that segment id by id (wavefront scans, joined in order).
+// The running sum is taken in id order at every level, so the pick differs from an exact
+// cumulative sum only where the target lies within rounding of a boundary.
+#define SAMPLE_WAVES (SAMPLE_THREADS / LLE_WAVE)
+#define SAMPLE_LINE 1024
+#define SAMPLE_MAX_SEGMENTS 2048
+#define SAMPLE_NONE 0x7fffffff
+
+__device__ __forceinline__ float wave_inclusive_scan(float v, int lane) {
+#pragma unroll
+    for (int o = 1; o < LLE_WAVE; o <<= 1) {
+        const float n = __shfl_up(v, o, LLE_WAVE);
+        if (lane >= o) v += n;
+    }
+    return v;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits,
                                                                      const float* __restrict__ temperature,
                                                                      const float* __restrict__ uniform,
                                                                      int32_t* __restrict__ out, int V) {
-    __shared__ float red[16];
-    __shared__ float s_part[SAMPLE_THREADS];
-    __shared__ int s_pick;
+    __shared__ float s_val[SAMPLE_WAVES];
+    __shared__ int s_idx[SAMPLE_WAVES];
+    __shared__ float s_seg[SAMPLE_MAX_SEGMENTS];
+    __shared__ float s_wave[SAMPLE_WAVES];
+    __shared__ float s_big, s_before, s_target;
+    __shared__ int s_big_i, s_seg_pick, s_pick, s_last;
     const float* row = logits + (int64_t)blockIdx.x * V;
     const float T = temperature[blockIdx.x];
-    const int t = threadIdx.x;
-    const int chunk = (V + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-    const int lo = min(V, t * chunk), hi = min(V, lo + chunk);
+    const int t = threadIdx.x, lane = t % LLE_WAVE, wave = t / LLE_WAVE;
 
     float mx = -INFINITY;
-    int mx_i = V;
-    for (int i = lo; i < hi; ++i)
-        if (row[i] > mx) {
-            mx = row[i];
+    int mx_i = SAMPLE_NONE;
+    for (int i = t; i < V; i += SAMPLE_THREADS) {  // ascending: the first maximum of this thread
+        const float v = row[i];
+        if (v > mx) {
+            mx = v;
             mx_i = i;
         }
-    const float big = block_max(mx, red);
-    if (T <= 0.f) {  // greedy: smallest index that reaches the maximum
-        if (t == 0) s_pick = V;
-        __syncthreads();
-        if (mx == big && mx_i < V) atomicMin(&s_pick, mx_i);
-        __syncthreads();
-        if (t == 0) out[blockIdx.x] = s_pick < V ? s_pick : 0;
+    }
+    block_argmax(mx, mx_i, s_val, s_idx);
+    if (t == 0) {
+        s_big = mx;
+        s_big_i = mx_i == SAMPLE_NONE ? 0 : mx_i;
+        s_pick = SAMPLE_NONE;
+        s_last = -1;
+    }
+    __syncthreads();
+    const float big = s_big;
+    if (T <= 0.f) {
+        if (t == 0) out[blockIdx.x] = s_big_i;
         return;
     }
     const float inv_t = 1.0f / T;
-    float part = 0.f;
-    for (int i = lo; i < hi; ++i) part += expf((row[i] - big) * inv_t);
-    s_part[t] = part;
-    __syncthreads();
-    if (t == 0) {
-        // sequential scan over 1024 partial sums: fixed order, once per row
-        float run = 0.f;
-        for (int k = 0; k < SAMPLE_THREADS; ++k) {
-            const float p = s_part[k];
-            s_part[k] = run;  // exclusive prefix
-            run += p;
-        }
-        red[0] = run;
-        s_pick = V;
-    }
-    __syncthreads();
-    const float total = red[0];
-    const float target = uniform[blockIdx.x] * total;
-    const float before = s_part[t];
-    if (lo < hi && target >= before && target < before + part) {
-        float run = before;
-        int pick = hi - 1;
-        for (int i = lo; i < hi; ++i) {
-            run += expf((row[i] - big) * inv_t);
-            if (run > target) {
-                pick = i;
-                break;
+    const int nlines = (V + SAMPLE_LINE - 1) / SAMPLE_LINE;
+    const int per_seg = (nlines + SAMPLE_MAX_SEGMENTS - 1) / SAMPLE_MAX_SEGMENTS;  // lines a segment
+    const int nseg = (nlines + per_seg - 1) / per_seg;
+    for (int seg = wave; seg < nseg; seg += SAMPLE_WAVES) {
+        float part = 0.f;
+        for (int g = 0; g < per_seg; ++g) {
+            const int64_t base = ((int64_t)seg * per_seg + g) * SAMPLE_LINE;
+            if (base >= V) break;
+            float v[SAMPLE_LINE / LLE_WAVE];
+#pragma unroll
+            for (int j = 0; j < SAMPLE_LINE / LLE_WAVE; ++j) {
+                const int64_t i = base + lane + LLE_WAVE * j;
+                v[j] = row[i < V ? i : V - 1];
             }
+#pragma unroll
+            for (int j = 0; j < SAMPLE_LINE / LLE_WAVE; ++j)
+                part += base + lane + LLE_WAVE * j < V ? expf((v[j] - big) * inv_t) : 0.f;
         }
-        atomicMin(&s_pick, pick);
+        part = wave_sum(part);
+        if (lane == 0) s_seg[seg] = part;
     }
     __syncthreads();
-    if (t == 0) out[blockIdx.x] = s_pick < V ? s_pick : V - 1;
+    if (wave == 0) {
+        // lane l owns the segments [l * each, (l + 1) * each)
+        const int each = (nseg + LLE_WAVE - 1) / LLE_WAVE;
+        float own = 0.f;
+        for (int k = 0; k < each; ++k) {
+            const int seg = lane * each + k;
+            own += seg < nseg ? s_seg[seg] : 0.f;
+        }
+        const float inclusive = wave_inclusive_scan(own, lane);
+        const float total = __shfl(inclusive, LLE_WAVE - 1, LLE_WAVE);
+        float before = __shfl_up(inclusive, 1, LLE_WAVE);
+        if (lane == 0) before = 0.f;
+        // a uniform number of exactly 1 (a double just below 1 rounds to it) would pick nothing
+        const float target = fminf(uniform[blockIdx.x], 0x1.fffffep-1f) * total;
+        int found = SAMPLE_NONE, last = -1;
+        float found_before = 0.f, last_before = 0.f, run = before;
+        for (int k = 0; k < each; ++k) {
+            const int seg = lane * each + k;
+            const float sum = seg < nseg ? s_seg[seg] : 0.f;
+            if (sum > 0.f) {
+                if (found == SAMPLE_NONE && run + sum > target) {
+                    found = seg;
+                    found_before = run;
+                }
+                last = seg;
+                last_before = run;
+            }
+            run += sum;
+        }
+        // the first lane that found one holds the first such segment; without any, the last
+        // segment that has weight at all
+        const unsigned long long have = __builtin_amdgcn_ballot_w64(found != SAMPLE_NONE);
+        const unsigned long long any = __builtin_amdgcn_ballot_w64(last >= 0);
+        int src = 0;
+        if (have)
+            src = __builtin_ctzll(have);
+        else if (any)
+            src = 63 - __builtin_clzll(any);
+        const int seg_pick = __shfl(have ? found : last, src, LLE_WAVE);
+        const float seg_before = __shfl(have ? found_before : last_before, src, LLE_WAVE);
+        if (lane == 0) {
+            s_seg_pick = (have || any) ? seg_pick : -1;
+            s_before = seg_before;
+            s_target = target;
+        }
+    }
+    __syncthreads();
+    const int seg = s_seg_pick;
+    if (seg < 0) {  // no id has weight (a row of NaN): the greedy pick
+        if (t == 0) out[blockIdx.x] = s_big_i;
+        return;
+    }
+    const float target = s_target;
+    float carry = s_before;
+    for (int g = 0; g < per_seg; ++g) {
+        const int64_t base = ((int64_t)seg * per_seg + g) * SAMPLE_LINE;
+        if (base >= V) break;
+        const int64_t i = base + t;
+        const float p = i < V ? expf((row[i] - big) * inv_t) : 0.f;
+        const float inclusive = wave_inclusive_scan(p, lane);
+        if (lane == LLE_WAVE - 1) s_wave[wave] = inclusive;
+        __syncthreads();
+        float ahead = 0.f, all = 0.f;
+#pragma unroll
+        for (int w = 0; w < SAMPLE_WAVES; ++w) {
+            if (w < wave) ahead += s_wave[w];
+            all += s_wave[w];
+        }
+        if (p > 0.f) {
+            if (carry + ahead + inclusive > target) atomicMin(&s_pick, (int)i);
+            atomicMax(&s_last, (int)i);
+        }
+        carry += all;
+        __syncthreads();
+    }
+    if (t == 0) out[blockIdx.x] = s_pick != SAMPLE_NONE ? s_pick : (s_last >= 0 ? s_last : s_big_i);
 }
 
 extern "C" int lle_sample_rows(const void* logits, const void* temperature, const void* uniform, void* out, int R,

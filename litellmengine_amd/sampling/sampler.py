@@ -15,6 +15,11 @@ from typing import List, Sequence
 import torch
 
 
+# the largest float32 below 1: a double just below 1 would round to 1.0 on its way to the kernel,
+# where no id's share of the running sum reaches
+MAX_UNIFORM = 1.0 - 2.0 ** -24
+
+
 class Sampler:
     def __init__(self, ops, device):
         self.ops = ops
@@ -29,6 +34,6 @@ class Sampler:
         if all(r.temperature <= 0.0 for r in requests):
             return self.ops.argmax(logits).tolist()
         temperature = [float(r.temperature) for r in requests]
-        uniform = [r.rng.random() if r.temperature > 0.0 else 0.0 for r in requests]
+        uniform = [min(r.rng.random(), MAX_UNIFORM) if r.temperature > 0.0 else 0.0 for r in requests]
         both = torch.tensor([temperature, uniform], dtype=torch.float32).to(self.device)
         return self.ops.sample(logits, both[0].contiguous(), both[1].contiguous()).tolist()

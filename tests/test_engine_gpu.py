@@ -11,7 +11,8 @@ from tests.tiny import PAGE_SIZES, make_model_dir, random_tokens
 
 pytestmark = pytest.mark.gpu
 
-TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+# about five times the worst error seen over dozens of seeds (float32 7e-7, bfloat16 7e-3 at these sizes)
+TOL = {"float32": 4e-6, "bfloat16": 2e-2}
 
 
 def make_runner(model_dir, dtype, page_size, num_pages, max_requests=4):
@@ -126,7 +127,7 @@ def test_qwen3_8b_layer_sizes(tmp_path):
     tokens = random_tokens(70, cfg.vocab_size, 5)
     want = plain.model_logits_fast(tokens, w, pcfg).double()
     scale = max(1.0, want.abs().max().item())
-    for dtype, tol in (("float32", 2e-4), ("bfloat16", 4e-2)):  # the oracle itself is float32 here
+    for dtype, tol in (("float32", 2e-5), ("bfloat16", 4e-2)):  # the oracle itself is float32 here
         runner = make_runner(d, dtype, 16, 8)
         for cuts in ([70], [38] + [1] * 32, [2, 17, 3, 30, 18]):
             got = run_cut(runner, tokens, cuts)

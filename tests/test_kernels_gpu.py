@@ -469,3 +469,29 @@ def test_argmax_and_sample(V):
                 lo, hi = sorted((got[r], want[r]))
                 assert abs(float(cdf[hi - 1]) - float(u[r])) < 1e-4 and hi - lo <= 2, (r, got[r], want[r])
     assert ops().sample(logits, temperature, u).cpu().tolist()[2] == 0
+    # a uniform number that rounds to 1.0 in float32 still picks an id that has weight: row 1 is
+    # peaked (all but 1e-17 of the weight on one id), so the running sum passes the target there
+    ones = torch.ones((6,), dtype=torch.float32).cuda()
+    assert ops().sample(logits, temperature, ones).cpu().tolist()[1] == V // 2
+    below = torch.full((6,), 1.0 - 2.0 ** -24, dtype=torch.float32).cuda()
+    assert ops().sample(logits, temperature, below).cpu().tolist()[1] == V // 2
+
+
+@pytest.mark.parametrize("V", [1024, 1025, 70000, 151936])
+def test_sample_every_region_of_the_row(V):
+    """Uniform numbers spread over [0, 1) against a flat-ish row: picks land in every segment
+    of the row and must agree with the exact running sum up to a boundary's rounding."""
+    g = torch.Generator().manual_seed(11)
+    R = 64
+    logits = (0.5 * torch.randn((R, V), generator=g)).cuda()
+    temperature = torch.full((R,), 0.9).cuda()
+    u = ((torch.arange(R, dtype=torch.float64) + 0.37) / R).float().cuda()
+    got = ops().sample(logits, temperature, u).cpu().tolist()
+    p = torch.softmax(logits.double().cpu() / 0.9, dim=1)
+    cdf = torch.cumsum(p, dim=1)
+    want = torch.searchsorted(cdf, u.double().cpu().unsqueeze(1) * cdf[:, -1:], right=True).squeeze(1).tolist()
+    assert len(set(w * 8 // V for w in want)) == 8  # every eighth of the row is hit
+    for r in range(R):
+        if got[r] != want[r]:
+            lo, hi = sorted((got[r], want[r]))
+            assert hi - lo <= 2 and abs(float(cdf[r, hi - 1]) - float(u[r])) < 1e-5, (r, got[r], want[r])
