@@ -276,6 +276,20 @@ class CacheManager:
             for group in self.groups:
                 group._lib.lle_pt_trim_many(group._h, n, slots, lens)
 
+    def shortfall(self, wants: Sequence[Tuple[int, int]]) -> List[int]:
+        """Per group: pages that `extend_many(wants)` needs minus the free ones (<= 0: they are there)."""
+        n, slots, lens, keep = self._arrays(wants)
+        out = []
+        for group in self.groups:
+            need = group._lib.lle_pt_pages_needed_many(group._h, n, slots, lens) if n else 0
+            out.append((group.pool.num_pages + 1 if need < 0 else need) - group.pool.num_free)
+        return out
+
+    def pages_held(self, slot: int) -> List[int]:
+        """Pages per group that the request in `slot` holds."""
+        self._check_live(slot)
+        return [len(g.held_pages(slot)) for g in self.groups]
+
     def free_pages(self) -> List[int]:
         return [g.pool.num_free for g in self.groups]
 

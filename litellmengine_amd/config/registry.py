@@ -9,7 +9,7 @@ call (the tests register a toy one without touching this package).
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Callable, Dict
+from typing import Any, Callable, Dict, Optional
 
 from .model_config import ConfigError, read_config_json
 
@@ -18,14 +18,17 @@ from .model_config import ConfigError, read_config_json
 class Architecture:
     name: str
     config_class: Any  # has from_dict(dict) and to_dict()
-    build: Callable[..., Any]  # build(config, build_context) -> models.decoder.DecoderLM
+    build: Callable[..., Any]  # build(config) -> models.decoder.DecoderLM
+    # chat_template(user_prompt, enable_thinking) -> the text that is tokenised for a text prompt;
+    # None: the prompt is tokenised as it is
+    chat_template: Optional[Callable[[str, bool], str]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_class, build) -> None:
-    _ARCHITECTURES[name] = Architecture(name, config_class, build)
+def register_architecture(name: str, config_class, build, chat_template=None) -> None:
+    _ARCHITECTURES[name] = Architecture(name, config_class, build, chat_template)
 
 
 def registered_architectures():
@@ -48,6 +51,10 @@ def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
     if not archs or not isinstance(archs, list):
         raise ConfigError("config.json has no `architectures` list to choose a model by")
     return get_architecture(str(archs[0]))
+
+
+def architecture_of_model_dir(model_dir: str) -> Architecture:
+    return architecture_of(read_config_json(model_dir))
 
 
 def load_config(model_dir: str):

@@ -12,6 +12,7 @@ import torch
 
 from ..parts.base import Prenormed
 from . import build
+from .limits import MAX_HEAD_DIM
 
 F32, BF16 = 0, 1
 _P = ctypes.c_void_p
@@ -51,7 +52,7 @@ def _dev(t: torch.Tensor, name: str, dtype=None) -> None:
 class HipOps:
     """The operations a model part may call.  One instance per process is enough."""
 
-    MAX_HEAD_DIM = 256
+    MAX_HEAD_DIM = MAX_HEAD_DIM
 
     def __init__(self):
         if not torch.cuda.is_available():

@@ -7,9 +7,10 @@ the worst case so that pages never run out
 `ensure_blocks` up to `main` (src/engine/block_table_manager.cpp:82-84).
 
 Here, every step:
- 1. requests that are decoding (one pending token) come first, then requests
-    with prompt tokens left, oldest first; each gets min(pending, prefill_chunk,
-    what is left of max_tokens_per_step) tokens;
+ 1. requests that are decoding (one pending token) come first, the one that was
+    served longest ago first (with a budget below the number of decoders they
+    take turns), then requests with prompt tokens left, oldest first; each gets
+    min(pending, prefill_chunk, what is left of max_tokens_per_step) tokens;
  2. if the pages for that are not there, the YOUNGEST running request is
     preempted: its pages and slot are given back, its cache is forgotten
     (cached_len = 0) and it waits at the FRONT of the queue to be recomputed
@@ -26,7 +27,9 @@ portions like any prompt; the reference feeds them one by one,
 src/engine/paged_generate_engine.cpp:133-141) or `release_request` ends it.
 Parked sessions come before running requests when pages run out: the one
 parked longest loses its cache first (it is recomputed whole if it is ever
-continued).
+continued).  A waiting request takes a parked session's cache only if that
+makes it fit: when the free pages and those of all parked sessions together
+are too few, nothing is evicted and the request goes on waiting.
 """
 from __future__ import annotations
 
@@ -66,6 +69,8 @@ class Scheduler:
         self._admissions = 0
         self.num_preemptions = 0
         self.num_evictions = 0  # parked sessions whose cache was taken
+        self._serve_clock = 0
+        self._last_served: Dict[int, int] = {}  # request id -> when tokens of it last ran (ticks of the clock)
 
     # -- adding ---------------------------------------------------------------------
     def add_request(self, prompt_ids: Sequence[int], max_new_tokens: int, eos_token_id: int = -1,
@@ -155,6 +160,16 @@ class Scheduler:
         self.num_evictions += 1
         return True
 
+    def _parked_pages_cover(self, short: Sequence[int]) -> bool:
+        """Whether the pages of all parked sessions make up for `short` (per group: pages
+        needed minus pages free)."""
+        if all(x <= 0 for x in short):
+            return True
+        have = [0] * len(short)
+        for r in self.parked:
+            have = [a + b for a, b in zip(have, self.cache.pages_held(r.slot))]
+        return all(x <= h for x, h in zip(short, have))
+
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
@@ -166,7 +181,8 @@ class Scheduler:
         budget = self.max_tokens_per_step
         chosen = None if only is None else set(only)
         mine = [r for r in self.running if chosen is None or r.request_id in chosen]
-        order = [r for r in mine if r.extend_len == 1] + [r for r in mine if r.extend_len > 1]
+        decoding = sorted((r for r in mine if r.extend_len == 1), key=lambda r: self._last_served.get(r.request_id, -1))
+        order = decoding + [r for r in mine if r.extend_len > 1]
         plan: List[Portion] = []
         for r in order:
             if budget == 0:
@@ -177,10 +193,12 @@ class Scheduler:
 
         preempted = False
         while plan and not self.cache.can_extend([(p.request.slot, p.start + p.num_tokens) for p in plan]):
+            if len(self.running) == 1 and not self._parked_pages_cover(
+                    self.cache.shortfall([(p.request.slot, p.start + p.num_tokens) for p in plan])):
+                raise OutOfPages("the only running request does not fit into the cache")  # nothing was evicted
             if self._evict_parked():
                 continue
-            if len(self.running) == 1:
-                raise OutOfPages("the only running request does not fit into the cache")
+            # the youngest of ALL running requests, whether this step runs it or not (`only`)
             victim = max(self.running, key=lambda r: r.admitted_at)
             self._preempt(victim)
             preempted = True
@@ -191,18 +209,24 @@ class Scheduler:
             r = next((w for w in self.waiting if chosen is None or w.request_id in chosen), None)
             if r is None:
                 break
-            if self.cache.num_free_slots == 0 and not self._evict_parked():
+            need_slot = self.cache.num_free_slots == 0
+            if need_slot and not self.parked:
                 break
             n = min(r.extend_len, self.prefill_chunk, budget)
-            slot = self.cache.admit()
-            wants = [(p.request.slot, p.start + p.num_tokens) for p in plan] + [(slot, n)]
-            while not self.cache.can_extend(wants) and self._evict_parked():
-                pass
-            if not self.cache.can_extend(wants):
-                self.cache.release(slot)
+            planned = [(p.request.slot, p.start + p.num_tokens) for p in plan]
+            short = [a + b for a, b in zip(self.cache.shortfall(planned), self.cache.pages_needed(None, n))]
+            if not self._parked_pages_cover(short):
+                # evicting every parked session would not make room: they keep their caches
                 if not self.running:
                     raise OutOfPages("the first waiting request does not fit into the empty cache")
                 break
+            if need_slot:
+                self._evict_parked()
+            slot = self.cache.admit()
+            wants = planned + [(slot, n)]
+            while not self.cache.can_extend(wants):
+                if not self._evict_parked():
+                    raise RuntimeError("the pages of parked sessions were counted but are not there")
             self.waiting.remove(r)
             r.slot = slot
             r.status = RequestStatus.RUNNING
@@ -211,6 +235,9 @@ class Scheduler:
             self.running.append(r)
             plan.append(Portion(r, 0, n, n == r.extend_len))
             budget -= n
+        for p in plan:  # a clock that ticks per portion: requests of one step keep their order for the next turn
+            self._serve_clock += 1
+            self._last_served[p.request.request_id] = self._serve_clock
         return plan
 
     def _preempt(self, r: Request) -> None:
@@ -236,6 +263,7 @@ class Scheduler:
                 r.append_token(next(it))
                 if r.finished:
                     self.running.remove(r)
+                    self._last_served.pop(r.request_id, None)
                     if r.keep_session:
                         self.parked.append(r)
                     else:

@@ -13,10 +13,14 @@ from .args import ArgsError, build_parser, parse_args, resolve_device
 from .token_ids import format_token_ids, parse_token_ids
 
 
-def qwen3_chat_template(user_prompt: str, enable_thinking: bool = False) -> str:
-    """src/tokenizer/qwen3_chat_template.cpp:7-24"""
-    text = "<|im_start|>user\n" + user_prompt + "<|im_end|>\n<|im_start|>assistant\n"
-    return text + ("<think>\n" if enable_thinking else "<think>\n\n</think>\n\n")
+def templated_prompt(model_dir: str, prompt: str, enable_thinking: bool = False) -> str:
+    """The text to tokenise for a user prompt: the chat template of the architecture that the
+    folder's config.json names (the reference applies Qwen3's to every model,
+    src/main.cpp:115-121), or the prompt itself for an architecture without one."""
+    from ..config.registry import architecture_of_model_dir
+
+    template = architecture_of_model_dir(model_dir).chat_template
+    return prompt if template is None else template(prompt, enable_thinking)
 
 
 def _load_tokenizer(model_dir: str):
@@ -49,7 +53,7 @@ def run(argv=None) -> int:
         print("\nInput token ids:\n  " + format_token_ids(input_ids), file=out)
     else:
         tokenizer = _load_tokenizer(args.model)
-        input_ids = tokenizer.encode(qwen3_chat_template(args.prompt, False), add_special_tokens=False).ids
+        input_ids = tokenizer.encode(templated_prompt(args.model, args.prompt, False), add_special_tokens=False).ids
         print("\nInput prompt:\n" + args.prompt, file=out)
         print("\nEncoded input token ids:\n  " + format_token_ids(input_ids), file=out)
     print(f"Input length: {len(input_ids)}", file=out)

@@ -7,30 +7,34 @@ and without it the engine is called in-process."""
 from __future__ import annotations
 
 import argparse
+import re
 import subprocess
 import sys
 from typing import List
 
-from .cli import qwen3_chat_template
+from .cli import templated_prompt
+from .token_ids import parse_token_ids
+
+# the output contract of the command line: the line "New token ids:", then a line with the ids
+_NEW_IDS = re.compile(r"^[ \t]*New token ids:[ \t]*\r?\n([^\r\n]*)", re.MULTILINE)
 
 
 def parse_new_token_ids(output: str) -> List[int]:
-    lines = output.splitlines()
-    for i, line in enumerate(lines):
-        if line.strip() == "New token ids:":
-            if i + 1 >= len(lines):
-                raise RuntimeError("Found 'New token ids:' but no ids line")
-            ids_line = lines[i + 1].strip()
-            if ids_line == "<none>":
-                return []
-            if not ids_line:
-                raise RuntimeError("Empty new token ids line")
-            return [int(x.strip()) for x in ids_line.split(",") if x.strip()]
-    raise RuntimeError("Could not find 'New token ids:' in the engine's output")
+    """The ids that the command line printed after `New token ids:` (`<none>`: no ids)."""
+    found = _NEW_IDS.search(output)
+    if found is None:
+        raise RuntimeError("the engine's output holds no 'New token ids:' line with ids after it")
+    ids = found.group(1).strip()
+    if ids == "<none>":
+        return []
+    try:
+        return parse_token_ids(ids)
+    except ValueError as e:
+        raise RuntimeError(f"the line after 'New token ids:' is no id list: {e}") from None
 
 
-def encode_prompt(tokenizer, prompt: str, use_chat_template: bool) -> List[int]:
-    text = qwen3_chat_template(prompt, enable_thinking=False) if use_chat_template else prompt
+def encode_prompt(tokenizer, model_dir: str, prompt: str, use_chat_template: bool) -> List[int]:
+    text = templated_prompt(model_dir, prompt, enable_thinking=False) if use_chat_template else prompt
     return list(tokenizer.encode(text, add_special_tokens=False).ids)
 
 
@@ -52,7 +56,7 @@ def main(argv=None) -> int:
     from tokenizers import Tokenizer
 
     tokenizer = Tokenizer.from_file(os.path.join(args.model, "tokenizer.json"))
-    input_ids = encode_prompt(tokenizer, args.prompt, not args.no_chat_template)
+    input_ids = encode_prompt(tokenizer, args.model, args.prompt, not args.no_chat_template)
     eos = args.eos_token_id
     if eos is None:
         eos = tokenizer.token_to_id("<|im_end|>")

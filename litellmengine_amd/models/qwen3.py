@@ -50,4 +50,11 @@ def build_qwen3(config: Qwen3Config) -> DecoderLM:
     )
 
 
-register_architecture(Qwen3Config.ARCHITECTURE, Qwen3Config, build_qwen3)
+def qwen3_chat_template(user_prompt: str, enable_thinking: bool = False) -> str:
+    """One user turn, then the start of the assistant's; with thinking off the empty
+    think block is already written (src/tokenizer/qwen3_chat_template.cpp:7-24)."""
+    text = "<|im_start|>user\n" + user_prompt + "<|im_end|>\n<|im_start|>assistant\n"
+    return text + ("<think>\n" if enable_thinking else "<think>\n\n</think>\n\n")
+
+
+register_architecture(Qwen3Config.ARCHITECTURE, Qwen3Config, build_qwen3, chat_template=qwen3_chat_template)

@@ -18,6 +18,7 @@ from typing import Dict, Optional
 
 import torch
 
+from ..csrc.limits import check_head_dim
 from ..weights.spec import INIT_NORM, TensorSpec
 from .base import BuildContext, KVCacheSpec, Mixer, PositionEncoding
 from .linear import Linear
@@ -41,6 +42,7 @@ class PagedAttention(Mixer):
     ):
         if num_q_heads % num_kv_heads:
             raise ValueError("num_q_heads must be a multiple of num_kv_heads")
+        check_head_dim(head_dim, getattr(position, "rotary_dim", 0))  # what no kernel takes is refused now, not at the first step
         self.prefix = prefix
         self.nq, self.nkv, self.d = num_q_heads, num_kv_heads, head_dim
         self.position = position

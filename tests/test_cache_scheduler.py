@@ -293,6 +293,84 @@ def test_no_admission_in_a_step_that_preempted():
     assert seen_preempt
 
 
+def run_plan(s, plan, token=7):
+    s.cache.extend_many([(p.request.slot, p.start + p.num_tokens) for p in plan])
+    for p in plan:
+        s.cache.commit(p.request.slot, p.start + p.num_tokens)
+    return s.update(plan, [token for p in plan if p.samples])
+
+
+def test_decoders_take_turns_when_the_budget_is_below_their_number():
+    s = Scheduler(manager(page_size=4, num_pages=32, max_requests=5), max_tokens_per_step=16)
+    reqs = [s.add_request([1, 2], 5) for _ in range(5)]
+    run_plan(s, s.schedule())  # all prompts in one step
+    assert all(r.extend_len == 1 for r in reqs)
+    s.max_tokens_per_step = 2
+    served = []
+    for _ in range(10):
+        plan = s.schedule()
+        assert len(plan) == 2 and all(p.num_tokens == 1 for p in plan)
+        served.append(sorted(p.request.request_id for p in plan))
+        run_plan(s, plan)
+        if not s.has_work():
+            break
+    # nobody waits for the head of the list to finish: within any three steps everyone ran
+    ids = [r.request_id for r in reqs]
+    for i in range(len(served) - 2):
+        window = set(served[i] + served[i + 1] + served[i + 2])
+        assert window >= {r for r in ids if not s.requests[r].finished or r in window}
+    counts = {r: sum(r in step for step in served[:5]) for r in ids}
+    assert max(counts.values()) - min(counts.values()) <= 1, counts
+
+
+def test_a_request_that_does_not_fit_leaves_parked_sessions_alone():
+    s = Scheduler(manager(page_size=4, num_pages=8, max_requests=4), max_tokens_per_step=64)
+    a = s.add_request(list(range(7)), 2, keep_session=True)   # parks with 2 pages
+    b = s.add_request(list(range(5)), 8)                      # runs on: up to 3 pages
+    while not a.finished:
+        run_plan(s, s.schedule())
+    assert s.parked == [a] and not b.finished
+    big = s.add_request(list(range(27)), 1)  # 7 pages: free + parked pages are too few while b runs
+    held_a = s.cache.pages_held(a.slot)
+    plan = s.schedule()
+    assert [p.request for p in plan] == [b]
+    assert s.num_evictions == 0 and s.parked == [a] and s.cache.pages_held(a.slot) == held_a
+    assert big.status is RequestStatus.WAITING
+    while not b.finished:
+        run_plan(s, s.schedule())
+    # now evicting the session makes room: it is evicted, and only now
+    while not big.finished:
+        run_plan(s, s.schedule())
+    assert s.num_evictions == 1 and a.slot == -1 and a.cached_len == 0
+
+
+def test_the_only_running_request_that_cannot_fit_raises_without_evicting():
+    s = Scheduler(manager("C", page_size=4, num_pages=6, max_requests=3), max_tokens_per_step=64, prefill_chunk=4)
+    a = s.add_request(list(range(6)), 1, keep_session=True)
+    while not a.finished:
+        run_plan(s, s.schedule())
+    assert s.parked == [a]
+    held = s.cache.pages_held(a.slot)
+    # fits the group with a window as far as add_request can tell, never the whole-cache group's pool:
+    # refused at once, the parked session untouched
+    with pytest.raises(ValueError, match="pages"):
+        s.add_request(list(range(40)), 1)
+    assert s.parked == [a] and s.cache.pages_held(a.slot) == held and s.num_evictions == 0
+
+
+def test_only_restricts_the_step_but_not_the_choice_of_the_victim():
+    s = Scheduler(manager(page_size=4, num_pages=4), max_tokens_per_step=64)
+    a = s.add_request(list(range(7)), 10)
+    b = s.add_request(list(range(4)), 8)
+    run_plan(s, s.schedule())  # both prompts: 2 + 1 pages of 4
+    assert a.slot >= 0 and b.slot >= 0
+    while s.cache.can_extend([(a.slot, a.cached_len + 1)]):
+        run_plan(s, s.schedule(only=[a.request_id]))
+        assert b.status is RequestStatus.RUNNING
+    plan = s.schedule(only=[a.request_id])  # a needs a page; b, the youngest, gives its pages although it does not run
+    assert [p.request for p in plan] == [a] and b.status is RequestStatus.WAITING and b.preemptions == 1
+
+
 # -- the step layout (csrc/host.cpp) ------------------------------------------------------
 def test_step_layout_matches_the_address_map():
     """Token ids, positions, requests, lengths, wanted rows and every token's page slot in

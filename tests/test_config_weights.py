@@ -170,3 +170,20 @@ def test_sharded_checkpoint(tmp_path):
     os.unlink(os.path.join(d, "model-00002-of-00002.safetensors"))
     with pytest.raises(WeightError, match="shard files that do not exist"):
         checkpoint_header(d)
+
+
+def test_sizes_that_no_kernel_takes_are_refused_when_the_model_is_built():
+    """src/model/qwen3.cpp:19-75 validates at construction; so does the builder here: a head the
+    attention kernels cannot hold is refused before any weight is read, naming the key."""
+    import pytest
+
+    from litellmengine_amd.config import ConfigError, Qwen3Config
+    from litellmengine_amd.config.registry import get_architecture
+    from tests.tiny import TINY_A
+
+    build = get_architecture("Qwen3ForCausalLM").build
+    build(Qwen3Config.from_dict(dict(TINY_A, head_dim=256)))
+    with pytest.raises(ValueError, match="head_dim 272"):
+        build(Qwen3Config.from_dict(dict(TINY_A, head_dim=272)))
+    with pytest.raises(ConfigError, match="head_dim must be even"):
+        Qwen3Config.from_dict(dict(TINY_A, head_dim=15))

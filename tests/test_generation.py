@@ -381,3 +381,29 @@ def test_sessions_on_the_gpu(tmp_path, dtype):
         assert r.generated == plain.generate_greedy(p + g + more, w, cfg, 5)
         eng.release_request(r)
     assert all(g.pool.num_held == 0 for g in eng.cache.groups)
+
+
+def test_chat_template_belongs_to_the_architecture(tmp_path):
+    """The command line asks the registry entry of the folder's architecture for the template
+    (src/tokenizer/qwen3_chat_template.cpp:7-24 for Qwen3); an architecture registered
+    without one gets its prompts as they are."""
+    import json
+    import os
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.config.registry import get_architecture, register_architecture
+    from litellmengine_amd.entrypoints.cli import templated_prompt
+
+    qwen = tmp_path / "qwen"
+    os.makedirs(qwen)
+    with open(qwen / "config.json", "w") as f:
+        json.dump(CONFIGS["A"], f)
+    assert templated_prompt(str(qwen), "Hi") == (
+        "<|im_start|>user\nHi<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n")
+    assert templated_prompt(str(qwen), "Hi", enable_thinking=True).endswith("<|im_start|>assistant\n<think>\n")
+    register_architecture("PlainPromptLM", Qwen3Config, get_architecture("Qwen3ForCausalLM").build)
+    other = tmp_path / "other"
+    os.makedirs(other)
+    with open(other / "config.json", "w") as f:
+        json.dump(dict(CONFIGS["A"], architectures=["PlainPromptLM"]), f)
+    assert templated_prompt(str(other), "Hi") == "Hi"
