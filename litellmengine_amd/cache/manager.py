@@ -15,7 +15,9 @@ no zero-filling of reused pages (lengths say what is valid).  Different:
    passed them;
  * mixers may ask for fixed-size state rows, zeroed at admission.
 
-Pool layout of a group: [layer, page, 2 (K, V), kv_head, page_size, head_dim].
+Pool layout of a group: [layer, page, elements of a page]; a page holds the fields of
+the mixers' per-token record one after the other (parts.base.CacheSpec).  For keys and
+values that is [layer, page, 2 (K, V), kv_head, page_size, head_dim], V transposed.
 """
 from __future__ import annotations
 
@@ -26,7 +28,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from ..parts.base import KVCacheSpec, StateSpec
+from ..parts.base import CacheSpec, StateSpec
 from .page_pool import OK, TOO_MANY_PAGES, OutOfPages, PagePool, PageTables
 
 
@@ -53,11 +55,11 @@ class _TableView:
 
 
 class CacheGroup:
-    """Pages, pool and block tables of the cache layers that share one KVCacheSpec.  The
+    """Pages, pool and block tables of the cache layers that share one CacheSpec.  The
     bookkeeping (free list, tables, what has not reached the device table yet) is the native
     host library's; the pool and the device table are tensors held here."""
 
-    def __init__(self, index: int, spec: KVCacheSpec, cache_ids: Sequence[int], page_size: int, num_pages: int,
+    def __init__(self, index: int, spec: CacheSpec, cache_ids: Sequence[int], page_size: int, num_pages: int,
                  max_requests: int, max_pages_per_request: int, dtype: torch.dtype, device: torch.device):
         self.index = index
         self.spec = spec
@@ -69,12 +71,21 @@ class CacheGroup:
         self.native = PageTables(num_pages, page_size, max_requests, max_pages_per_request, spec.window)
         self._lib, self._h = self.native.lib, self.native.handle
         self.pool = PagePool(num_pages, self.native)
-        self.kv = torch.zeros(
-            (len(self.cache_ids), num_pages, 2, spec.num_kv_heads, page_size, spec.head_dim), dtype=dtype, device=device
-        )
-        # per request slot: logical page -> physical page (-1 once the window has passed it)
+        # One page more than the pool hands out: page `num_pages` is never written (it stays zero)
+        # and is what the spare table row below points at.  A page is flat: the record's fields
+        # one after the other, each for all tokens of the page.
+        self.page_elems = page_size * spec.elems_per_token
+        self.data = torch.zeros((len(self.cache_ids), num_pages + 1, self.page_elems), dtype=dtype, device=device)
+        # keys and values in the attention kernels' layout: the same memory as
+        # [layer, page, 2 (K, V), kv_head, page_size, head_dim]
+        pair = spec.keys_and_values()
+        self.kv = None if pair is None else self.data.view(
+            len(self.cache_ids), num_pages + 1, 2, pair[0], page_size, pair[1])
+        # per request slot: logical page -> physical page (-1 once the window has passed it);
+        # row `max_requests` belongs to no request: rows that pad a batch read one key through it
         self.tables = _TableView(self)
-        self.block_table = torch.full((max_requests, max_pages_per_request), -1, dtype=torch.int32, device=device)
+        self.block_table = torch.full((max_requests + 1, max_pages_per_request), -1, dtype=torch.int32, device=device)
+        self.block_table[max_requests, 0] = num_pages
         self.slot_mapping: Optional[torch.Tensor] = None  # int32 [N] of the step being run
 
     def pages_for(self, length: int) -> int:
@@ -132,14 +143,30 @@ class CacheGroup:
 
 @dataclasses.dataclass
 class LayerCache:
-    """What the mixer of one plan entry gets: the pages of its cache layer
-    [page, 2, kv_head, page_size, head_dim], its group (block table and the
-    step's slot mapping), whether it writes, and its state rows [slot, ...]."""
+    """What the mixer of one plan entry gets: the pages of its cache layer (`pages`,
+    flat [page, elements]; `kv`, the same memory as [page, 2, kv_head, page_size,
+    head_dim] when the record is a key/value pair; `field(name)` for any record), its
+    group (block table and the step's slot mapping), whether it writes, and its state
+    rows [slot, ...]."""
 
     group: Optional[CacheGroup]
     kv: Optional[torch.Tensor]
     writes: bool
     state: Optional[torch.Tensor]
+    pages: Optional[torch.Tensor] = None
+
+    def field(self, name: str) -> torch.Tensor:
+        """The pages' share of one field of the record: [page, head, page_size, width], or
+        [page, head, width, page_size] for a transposed field (a view, no copy)."""
+        group = self.group
+        at = 0
+        for f in group.spec.fields:
+            n = f.elems_per_token * group.page_size
+            if f.name == name:
+                shape = (f.num_heads, f.width, group.page_size) if f.transposed else (f.num_heads, group.page_size, f.width)
+                return self.pages[:, at : at + n].unflatten(1, shape)
+            at += n
+        raise KeyError(f"the cache record has no field {name!r}")
 
 
 class CacheManager:
@@ -152,11 +179,12 @@ class CacheManager:
         device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
+        self.pad_slot = max_requests  # the table row (of every group) that padding rows of a batch read
         self.device = device
         self.dtype = dtype
         max_pages_per_request = max_pages_per_request or num_pages
 
-        by_spec: Dict[KVCacheSpec, List[int]] = {}
+        by_spec: Dict[CacheSpec, List[int]] = {}
         for cache_id, mixer in sorted(model.cache_layers().items()):
             spec = mixer.cache_spec()
             if spec is not None:
@@ -180,7 +208,8 @@ class CacheManager:
                 self.states[entry.cache] = torch.zeros((max_requests,) + tuple(sspec.shape), dtype=sspec.dtype, device=device)
             group, n = where.get(entry.cache, (None, 0))
             self._layers.append(
-                LayerCache(group, None if group is None else group.kv[n], entry.writes, self.states.get(entry.cache))
+                LayerCache(group, None if group is None or group.kv is None else group.kv[n], entry.writes,
+                           self.states.get(entry.cache), None if group is None else group.data[n])
             )
 
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))

@@ -233,10 +233,15 @@ void lle_pt_take_pending(void* h, int32_t* index, int32_t* pages) {
 // out: token ids [N], positions [N], request of each token [N], slots [S], first row of each
 // request and N [S + 1], cached length after the step [S], wanted rows [R], then for every group
 // the page slot of every token [N].  *info: the offending index when a code is returned.
+//
+// `pad` > 0 appends that many requests that stand for nobody (a batch padded to a size for which a
+// graph exists): one token each (id 0, position 0, cached length 1), block-table row `pad_slot`
+// (a row that points at a page nobody writes), page slot -1 (nothing is written).  The sizes above
+// then count them: N + pad tokens, S + pad requests; `logit_rows` may name their rows.
 int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int32_t* q_len, const int32_t* tokens,
-                    int vocab_size, int R, const int32_t* logit_rows, int G, void* const* groups, int32_t* out,
-                    int64_t* info) {
-    if (S <= 0 || R < 0 || G < 0) return LLE_HOST_BAD_ARGUMENT;
+                    int vocab_size, int R, const int32_t* logit_rows, int G, void* const* groups, int pad,
+                    int pad_slot, int32_t* out, int64_t* info) {
+    if (S <= 0 || R < 0 || G < 0 || pad < 0 || (pad > 0 && pad_slot < 0)) return LLE_HOST_BAD_ARGUMENT;
     int64_t N = 0;
     for (int s = 0; s < S; ++s) {
         if (q_len[s] <= 0 || past[s] < 0) {
@@ -251,7 +256,7 @@ int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int3
             return LLE_HOST_BAD_TOKEN;
         }
     for (int r = 0; r < R; ++r)
-        if (logit_rows[r] < 0 || logit_rows[r] >= N) {
+        if (logit_rows[r] < 0 || logit_rows[r] >= N + pad) {
             *info = r;
             return LLE_HOST_BAD_ARGUMENT;
         }
@@ -268,13 +273,15 @@ int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int3
                 }
         }
     }
+    const int64_t NP = N + pad;
+    const int SP = S + pad;
     int32_t* token_ids = out;
-    int32_t* positions = token_ids + N;
-    int32_t* token_seq = positions + N;
-    int32_t* seq_slots = token_seq + N;
-    int32_t* cu_tokens = seq_slots + S;
-    int32_t* kv_lens = cu_tokens + S + 1;
-    int32_t* rows = kv_lens + S;
+    int32_t* positions = token_ids + NP;
+    int32_t* token_seq = positions + NP;
+    int32_t* seq_slots = token_seq + NP;
+    int32_t* cu_tokens = seq_slots + SP;
+    int32_t* kv_lens = cu_tokens + SP + 1;
+    int32_t* rows = kv_lens + SP;
     int32_t* mapping = rows + R;
     std::copy(tokens, tokens + N, token_ids);
     int64_t at = 0;
@@ -288,12 +295,20 @@ int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int3
         }
         at += q_len[s];
     }
-    cu_tokens[S] = (int32_t)N;
+    for (int i = 0; i < pad; ++i) {
+        token_ids[N + i] = 0;
+        positions[N + i] = 0;
+        token_seq[N + i] = S + i;
+        seq_slots[S + i] = pad_slot;
+        cu_tokens[S + i] = (int32_t)(N + i);
+        kv_lens[S + i] = 1;
+    }
+    cu_tokens[SP] = (int32_t)NP;
     std::copy(logit_rows, logit_rows + R, rows);
     for (int g = 0; g < G; ++g) {
         const PageTables* t = pt(groups[g]);
         const int P = t->page_size;
-        int32_t* m = mapping + (int64_t)g * N;
+        int32_t* m = mapping + (int64_t)g * NP;
         at = 0;
         for (int s = 0; s < S; ++s) {
             const std::vector<int32_t>& table = t->tables[slots[s]];
@@ -303,6 +318,7 @@ int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int3
             }
             at += q_len[s];
         }
+        for (int i = 0; i < pad; ++i) m[N + i] = -1;
     }
     return LLE_HOST_OK;
 }

@@ -93,12 +93,15 @@ _staging = _Staging()
 
 
 def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, vocab_size: int = 0,
-                device=None) -> StepLayout:
+                device=None, pad_to: int = 0) -> StepLayout:
     """Lay the entries out flat and compute every token's page slot in every cache
     group (csrc/host.cpp does both).  Pages for the new lengths must already be there.
     `all_rows` asks for the logits of every row whatever the entries want; with
-    `vocab_size` token ids outside [0, vocab_size) are refused."""
+    `vocab_size` token ids outside [0, vocab_size) are refused.  `pad_to` fills the batch
+    up to that many requests with single tokens that stand for nobody: they read the
+    cache's spare table row and page (`cache.pad_slot`) and write nothing."""
     S = len(entries)
+    pad = max(0, pad_to - S)
     slots = array("i", (e.slot for e in entries))
     past = array("i", (cache.length(e.slot) for e in entries))
     q_len = array("i", (len(e.tokens) for e in entries))
@@ -114,22 +117,28 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
             rows.extend(start + int(w) for w in e.want)
         seqs.append(SeqInfo(e.slot, start, n, p))
         start += n
-    N, R, G = start, len(rows), len(cache.groups)
+    N, G = start, len(cache.groups)
+    if pad:
+        if all_rows:
+            rows.extend(range(N, N + pad))
+        seqs.extend(SeqInfo(cache.pad_slot, N + i, 1, 0) for i in range(pad))
+    R = len(rows)
     pinned = device is not None and torch.device(device).type == "cuda"
-    host = _staging.get(3 * N + 3 * S + 1 + R + G * N, pinned)
+    host = _staging.get(3 * (N + pad) + 3 * (S + pad) + 1 + R + G * (N + pad), pinned)
     lib = host_library()
     handles = (ctypes.c_void_p * max(1, G))(*[g.native.handle for g in cache.groups])
     info = ctypes.c_int64(0)
     address = lambda a: a.buffer_info()[0]
     code = lib.lle_layout_step(S, address(slots), address(past), address(q_len), address(tokens), int(vocab_size), R,
-                               address(rows), G, handles, host.data_ptr(), ctypes.byref(info))
+                               address(rows), G, handles, pad, cache.pad_slot if pad else 0, host.data_ptr(),
+                               ctypes.byref(info))
     if code == BAD_TOKEN:
         raise ValueError(f"token id {tokens[info.value]} outside [0, {vocab_size})")
     if code == NO_PAGE_AT_POSITION:
         raise IndexError(f"position {info.value} has no page: the cache was not extended for this step")
     if code != 0:
         raise ValueError(f"the step cannot be laid out: {lib.lle_error_string(code).decode()} (at {info.value})")
-    return StepLayout(host, N, S, R, G, seqs, max(p + n for p, n in zip(past, q_len)))
+    return StepLayout(host, N + pad, S + pad, R, G, seqs, max(p + n for p, n in zip(past, q_len)))
 
 
 def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:

@@ -10,13 +10,19 @@ are written to their pages first, then every token attends through the block
 table (src/model/qwen3.cpp:464-481 before :498-557).
 
 Steps that hold single tokens only (decoding) are launch-bound, so they are
-captured once per (batch size, context bucket) into a HIP graph and replayed:
-the step's integer arrays are copied into the graph's fixed buffer, the block
-tables are updated outside the graph, and the same kernels run.  Models whose
-mixers need the host-side view of the batch are stepped without graphs.
+captured into HIP graphs and replayed: the step's integer arrays are copied
+into the graph's fixed buffer, the block tables are updated outside the graph,
+and the same kernels run.  There is one graph per (batch bucket, context
+bucket): a batch is filled up to the next of a few sizes with rows that stand
+for nobody (they read one key of a page that is never written, write nothing,
+and their logits are dropped), so a batch whose requests finish one by one
+walks through a handful of graphs instead of one per size; the graphs used
+least recently are dropped beyond MAX_GRAPHS.  Models whose mixers need the
+host-side view of the batch are stepped without graphs.
 """
 from __future__ import annotations
 
+import collections
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -35,6 +41,8 @@ class _DecodeGraph:
 class ModelRunner:
     MAX_GRAPH_BATCH = 256
     MIN_CONTEXT_BUCKET = 256
+    BATCH_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+    MAX_GRAPHS = 32  # each keeps float32 logits [batch bucket, vocabulary] alive
 
     def __init__(self, model, cache: CacheManager, use_graphs: Optional[bool] = None):
         self.model = model
@@ -46,8 +54,9 @@ class ModelRunner:
         if use_graphs is None:
             use_graphs = self.device.type == "cuda"
         self.use_graphs = bool(use_graphs) and graph_safe and self.device.type == "cuda"
-        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._graphs: "collections.OrderedDict[Tuple[int, int], _DecodeGraph]" = collections.OrderedDict()
         self._graph_pool = None
+        self.num_captures = 0
 
     # requests ------------------------------------------------------------------
     def admit(self) -> int:
@@ -103,25 +112,31 @@ class ModelRunner:
     # decoding through a captured graph ---------------------------------------------------
     def _graph_step(self, entries: Sequence[StepEntry], borrow: bool) -> torch.Tensor:
         cache = self.cache
-        layout = layout_step(entries, cache, all_rows=True, vocab_size=self.vocab_size, device=self.device)
+        batch = next(b for b in self.BATCH_BUCKETS if b >= len(entries))
+        layout = layout_step(entries, cache, all_rows=True, vocab_size=self.vocab_size, device=self.device,
+                             pad_to=batch)
         apply_table_updates(cache, self.device)
         bucket = self.MIN_CONTEXT_BUCKET
         while bucket < layout.max_kv_len:
             bucket *= 2
         host = layout.host
-        key = (layout.num_seqs, bucket)
+        key = (batch, bucket)
         g = self._graphs.get(key)
         if g is None:
+            while len(self._graphs) >= self.MAX_GRAPHS:
+                self._graphs.popitem(last=False)  # the one used least recently
             g = self._capture(layout, host, bucket)
             self._graphs[key] = g
+            self.num_captures += 1
         else:
+            self._graphs.move_to_end(key)
             g.buf.copy_(host)
-        # the slot mappings of the groups must point into this graph's buffer while it runs
-        g.graph.replay()
+        g.graph.replay()  # its kernels read the buffer that the capture saw: g.buf
         logits = g.logits
         rows = [i for i, e in enumerate(entries) if len(e.want) > 0]
         if len(rows) != len(entries):
             return logits[torch.tensor(rows, dtype=torch.long, device=self.device)] if rows else logits[:0].clone()
+        logits = logits[: len(entries)]
         return logits if borrow else logits.clone()
 
     def _capture(self, layout: StepLayout, host: torch.Tensor, bucket: int) -> _DecodeGraph:

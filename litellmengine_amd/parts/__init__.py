@@ -1,5 +1,5 @@
 from .attention import PagedAttention
-from .base import Block, BuildContext, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part, PositionEncoding, Prenormed, StateSpec
+from .base import Block, BuildContext, CacheField, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part, PositionEncoding, Prenormed, StateSpec
 from .block import PreNormBlock
 from .embedding import Embedding
 from .feed_forward import GatedMLP
@@ -8,7 +8,7 @@ from .norm import RMSNorm
 from .position import NoPositionEncoding, RotaryHalfSplit
 
 __all__ = [
-    "Block", "BuildContext", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
+    "Block", "BuildContext", "CacheField", "CacheSpec", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
     "NoPositionEncoding", "Norm", "NormFold", "PagedAttention", "Part", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec",
 ]

@@ -20,7 +20,7 @@ import torch
 
 from ..csrc.limits import check_head_dim
 from ..weights.spec import INIT_NORM, TensorSpec
-from .base import BuildContext, KVCacheSpec, Mixer, PositionEncoding
+from .base import BuildContext, CacheSpec, KVCacheSpec, Mixer, PositionEncoding
 from .linear import Linear
 
 
@@ -58,7 +58,7 @@ class PagedAttention(Mixer):
         self.q_norm_w = None
         self.k_norm_w = None
 
-    def cache_spec(self) -> KVCacheSpec:
+    def cache_spec(self) -> CacheSpec:
         return KVCacheSpec(self.nkv, self.d, self.window)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:

@@ -29,13 +29,58 @@ class BuildContext:
 
 
 @dataclasses.dataclass(frozen=True)
-class KVCacheSpec:
-    """Per-token cache need of a mixer: keys and values of `num_kv_heads` heads of
-    `head_dim`; with a `window` only the last `window` positions stay needed."""
+class CacheField:
+    """One named part of what a mixer keeps per token: `num_heads` vectors of `width`
+    elements.  Inside a page the vectors of a head lie token after token
+    ([head][token][width]) or, `transposed`, element after element ([head][width][token])."""
 
-    num_kv_heads: int
-    head_dim: int
+    name: str
+    num_heads: int
+    width: int
+    transposed: bool = False
+
+    @property
+    def elems_per_token(self) -> int:
+        return self.num_heads * self.width
+
+
+@dataclasses.dataclass(frozen=True)
+class CacheSpec:
+    """Per-token cache need of a mixer: a record of named fields for every token.  A page
+    holds the fields one after the other, each for all of the page's tokens.  With a
+    `window` only the last `window` positions stay needed and pages behind it are given back.
+    Mixers with equal specs share a group of pages and block tables."""
+
+    fields: Tuple[CacheField, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [f.name for f in self.fields]
+        if not names or len(set(names)) != len(names):
+            raise ValueError("a cache record needs at least one field, and every field a name of its own")
+        for f in self.fields:
+            if f.num_heads <= 0 or f.width <= 0:
+                raise ValueError(f"cache field {f.name!r} needs positive sizes")
+
+    @property
+    def elems_per_token(self) -> int:
+        return sum(f.elems_per_token for f in self.fields)
+
+    def keys_and_values(self) -> Optional[Tuple[int, int]]:
+        """(kv heads, head size) if the record is the pair that the attention kernels read:
+        keys token after token, then values transposed, of the same shape; else None."""
+        if len(self.fields) != 2:
+            return None
+        k, v = self.fields
+        if k.transposed or not v.transposed or (k.num_heads, k.width) != (v.num_heads, v.width):
+            return None
+        return k.num_heads, k.width
+
+
+def KVCacheSpec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> CacheSpec:
+    """Keys and values of `num_kv_heads` heads of `head_dim`, in the layout the attention
+    kernels read: K as [head][token][d], V transposed as [head][d][token]."""
+    return CacheSpec((CacheField("k", num_kv_heads, head_dim), CacheField("v", num_kv_heads, head_dim, True)), window)
 
 
 @dataclasses.dataclass(frozen=True)
@@ -124,7 +169,7 @@ class Mixer(Part):
     # a keyword `fold` (a NormFold for its last product, whose Prenormed it then returns).
     folds_norm = False
 
-    def cache_spec(self) -> Optional[KVCacheSpec]:
+    def cache_spec(self) -> Optional[CacheSpec]:
         return None
 
     def state_spec(self) -> Optional[StateSpec]:

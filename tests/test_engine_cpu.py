@@ -85,3 +85,18 @@ def test_page_size_and_batch_order_do_not_matter(tmp_path):
     for page_size, reverse in ((1, False), (16, False), (4, True), (16, True)):
         for g, b in zip(run(page_size, reverse), base):
             assert (g - b).abs().max().item() < 1e-5, (page_size, reverse)
+
+
+def test_a_cache_record_that_is_no_key_value_pair_on_the_cpu(monkeypatch):
+    """The latent-vector mixer of tests/test_parts_gpu.py (a per-token cache record with one
+    field, with and without a window) through the same cache manager and step function, with
+    the substitute kernels."""
+    import torch
+
+    import tests.test_parts_gpu as parts_tests
+    from litellmengine_amd.parts.base import BuildContext
+    from tests.torch_ops import TorchOps
+
+    monkeypatch.setattr(parts_tests, "make_context",
+                        lambda dtype: BuildContext(dtype=dtype, device=torch.device("cpu"), ops=TorchOps()))
+    parts_tests.test_a_cache_record_that_is_no_key_value_pair(torch.float32)

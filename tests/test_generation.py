@@ -407,3 +407,26 @@ def test_chat_template_belongs_to_the_architecture(tmp_path):
     with open(other / "config.json", "w") as f:
         json.dump(dict(CONFIGS["A"], architectures=["PlainPromptLM"]), f)
     assert templated_prompt(str(other), "Hi") == "Hi"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_shrinking_batch_walks_through_few_graphs(tmp_path, dtype):
+    """Thirteen requests that finish one after the other: the decode batch shrinks from 13 to 1,
+    padded to 16, 8, 4, 2, 1 with rows that stand for nobody, so five graphs are captured, not
+    thirteen; every request generates what the plain model generates."""
+    d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    model = load_model(d, dtype)
+    eng = LLMEngine(model, page_size=16, num_pages=13 * 4, max_requests=13, max_tokens_per_step=512)
+    prompts = [random_tokens(5 + 2 * i, 419, 300 + i) for i in range(13)]
+    reqs = [eng.add_request(p, 2 + i) for i, p in enumerate(prompts)]  # the i-th finishes after 2 + i tokens
+    eng.run_until_finished()
+    assert eng.runner.use_graphs and eng.runner.num_captures <= 5, eng.runner.num_captures
+    assert sorted(k[0] for k in eng.runner._graphs) == [1, 2, 4, 8, 16]
+    for r, p in zip(reqs, prompts):
+        if dtype == "float32":
+            assert r.generated == plain.generate_greedy(p, w, cfg, r.max_new_tokens)
+        else:
+            assert len(r.generated) == r.max_new_tokens and near_greedy(p, r.generated, w, cfg, 8e-2)
+    assert all(g.pool.num_held == 0 for g in eng.cache.groups)

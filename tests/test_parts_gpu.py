@@ -313,3 +313,91 @@ def test_toy_architecture_registers_builds_and_steps(dtype):
     assert s2 == sx
     again = runner.step([StepEntry(s2, seqs["y"], list(range(13)))]).cpu()
     assert (again.double() - want["y"]).abs().max() < TOL[dtype]
+
+
+# ---------------------------------------------------------------------------------------
+# a mixer whose per-token cache is no key/value pair: one latent vector a token
+# ---------------------------------------------------------------------------------------
+class LatentMeanMixer(Mixer):
+    """c_t = W_down x_t is cached (one vector of `rank` elements per token, in pages);
+    y_t = W_up mean(c_0 .. c_t), the mean read back from the pages through the block table."""
+
+    def __init__(self, prefix, hidden, rank, window=None):
+        self.prefix, self.hidden, self.rank, self.window = prefix, hidden, rank, window
+
+    def tensor_specs(self):
+        return {self.prefix + "down": TensorSpec((self.rank, self.hidden)),
+                self.prefix + "up": TensorSpec((self.hidden, self.rank))}
+
+    def cache_spec(self):
+        from litellmengine_amd.parts import CacheField, CacheSpec
+
+        return CacheSpec((CacheField("latent", 1, self.rank),), self.window)
+
+    def bind(self, weights, ctx):
+        self.ctx = ctx
+        self.down = weights[self.prefix + "down"].to(ctx.dtype).contiguous()
+        self.up = weights[self.prefix + "up"].to(ctx.dtype).contiguous()
+
+    def forward(self, x, step, cache):
+        c = self.ctx.ops.linear(x, self.down)
+        pages = cache.field("latent")  # [page, 1, page_size, rank]
+        P = pages.shape[2]
+        if cache.writes:
+            where = cache.group.slot_mapping.long()
+            pages[where // P, 0, where % P] = c
+        y = torch.empty_like(c)
+        for q in step.seqs:
+            table = cache.group.block_table[q.slot].long()
+            for t in range(q.q_len):
+                pos = q.past_len + t
+                lo = max(0, pos - self.window + 1) if self.window else 0
+                at = torch.arange(lo, pos + 1, device=x.device)
+                seen = pages[table[at // P], 0, at % P].float()
+                y[q.q_start + t] = seen.mean(dim=0).to(y.dtype)
+        return self.ctx.ops.linear(y, self.up)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_cache_record_that_is_no_key_value_pair(dtype):
+    """The cache manager pages whatever record a mixer declares: here one latent vector per
+    token, once for all positions and once behind a window (two groups: pages of the second
+    are given back and used again).  Portions, single tokens and a second request in pages
+    that the first has freed, against the running mean computed whole."""
+    hidden, rank, window, page = 40, 12, 7, 4
+    mixers = [LatentMeanMixer("l0.mix.", hidden, rank), LatentMeanMixer("l1.mix.", hidden, rank, window)]
+    blocks = [PreNormBlock(RMSNorm(f"l{i}.n1", hidden, 1e-5), m, RMSNorm(f"l{i}.n2", hidden, 1e-5),
+                           GatedMLP(f"l{i}.mlp.", hidden, 56)) for i, m in enumerate(mixers)]
+    model = DecoderLM(None, Embedding("emb", 61, hidden), blocks, [PlanEntry(0), PlanEntry(1)],
+                      RMSNorm("fn", hidden, 1e-5), Linear(["head"], hidden, [61]), tied_head=False)
+    ctx, w = bound(model, dtype, seed=4)
+    model.ctx = ctx
+    cache = CacheManager(model, page_size=page, num_pages=8, max_requests=2, dtype=dtype, device=ctx.device)
+    assert len(cache.groups) == 2 and all(g.kv is None for g in cache.groups)
+    assert cache.groups[0].data.shape == (1, 8 + 1, page * rank)
+
+    def whole(ids):
+        T = len(ids)
+        h = plain.embedding(ids, w["emb"])
+        for i, win in enumerate((None, window)):
+            c = plain.linear(plain.rms_norm(h, w[f"l{i}.n1"], 1e-5), w[f"l{i}.mix.down"])
+            y = torch.stack([c[max(0, t - win + 1) if win else 0 : t + 1].mean(dim=0) for t in range(T)])
+            h = h + plain.linear(y, w[f"l{i}.mix.up"])
+            h = h + plain.gated_mlp(plain.rms_norm(h, w[f"l{i}.n2"], 1e-5), w[f"l{i}.mlp.gate_proj.weight"],
+                                    w[f"l{i}.mlp.up_proj.weight"], w[f"l{i}.mlp.down_proj.weight"])
+        return plain.fast_linear(plain.rms_norm(h, w["fn"], 1e-5), w["head"])
+
+    runner = ModelRunner(model, cache)
+    assert not runner.use_graphs  # the mixer reads the host's view of the batch
+    for seed, cuts in ((1, [9, 1, 1, 6, 1, 9]), (2, [2, 13, 1, 1, 1, 5])):
+        ids = random_tokens(sum(cuts), 61, seed)
+        want = whole(ids)
+        slot, at, got = runner.admit(), 0, []
+        for n in cuts:
+            got.append(runner.step([StepEntry(slot, ids[at : at + n], list(range(n)))]).cpu())
+            at += n
+        err = (torch.cat(got).double() - want).abs().max().item()
+        assert err < TOL[dtype], (seed, err)
+        assert cache.groups[1].pool.num_held <= (window + page - 1) // page + 1  # the window let pages go
+        runner.release(slot)
+    assert all(g.pool.num_held == 0 for g in cache.groups)
