@@ -123,6 +123,47 @@ def time_prefill(model, cfg, tokens, repeats=3):
     return best
 
 
+def measure_peaks(dtype):
+    """What this machine reaches on kernels that do nothing else: (bytes/s of a kernel that only
+    reads 4 GiB from HBM, flops/s of a kernel that only issues matrix instructions of `dtype`
+    on registers).  The rooflines are given against the published peaks and against these."""
+    import torch
+
+    from litellmengine_amd.csrc.ops import default_ops
+
+    ops = default_ops()
+
+    def timed(launch):
+        launch()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            launch()
+            end.record()
+            end.synchronize()
+            dt = start.elapsed_time(end) * 1e-3
+            best = dt if best is None else min(best, dt)
+        return best
+
+    data = torch.empty(1 << 30, dtype=torch.int32, device="cuda")  # 4 GiB: far more than the caches hold
+    data.fill_(1)
+    nbytes = data.numel() * 4
+    read = max(nbytes / timed(lambda b=b: ops.probe_read_stream(data, b)) for b in (256, 16384, 65536))
+    del data
+    torch.cuda.empty_cache()
+    tdtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    flops = [0.0]
+
+    def mfma():
+        flops[0] = ops.probe_mfma(tdtype, 8 * units, 4000)
+
+    seconds = timed(mfma)
+    return read, flops[0] / seconds
+
+
 def flat_config(cfg, full_layers, **more):
     d = {"layers": cfg.num_hidden_layers, "layers_of_full_model": full_layers, "hidden": cfg.hidden_size,
          "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
@@ -304,6 +345,11 @@ def main():
         pt = time_prefill(model, cfg, PREFILL_TOKENS)
         line["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
                            "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MFMA_PEAK[short], 4)}
+        read_peak, mfma_peak = measure_peaks(args.dtype)
+        line["roofline"]["measured_peak"] = round(read_peak / 1e9, 1)
+        line["roofline"]["frac_of_measured"] = round(achieved / read_peak, 4)
+        line["prefill"]["measured_peak_tflops"] = round(mfma_peak / 1e12, 1)
+        line["prefill"]["frac_of_measured"] = round(prefill_flops(cfg, PREFILL_TOKENS) / pt / mfma_peak, 4)
         points = {}
         for b in (1, 64):
             s = max(8, args.steps // 2)

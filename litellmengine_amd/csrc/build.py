@@ -32,6 +32,7 @@ LIBRARIES: Dict[str, List[str]] = {
     "attention": ["attention.hip"],
     "gemm": ["gemm.hip"],
     "sampling": ["sampling.hip"],
+    "probe": ["probe.hip"],
 }
 # libraries without GPU code: compiled with the host's C++ compiler
 HOST_LIBRARIES: Dict[str, List[str]] = {"host": ["host.cpp"]}

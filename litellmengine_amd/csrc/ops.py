@@ -487,6 +487,21 @@ class HipOps:
         return out
 
 
+    # -- measured peaks (the benchmark's rooflines) ---------------------------------------------
+    def probe_read_stream(self, data: torch.Tensor, blocks: int) -> None:
+        """Launch a kernel that only reads `data` (any type, a multiple of 16 bytes), `blocks` workgroups."""
+        _dev(data, "data")
+        nbytes = data.numel() * data.element_size()
+        _need(nbytes % 16 == 0 and nbytes > 0, "the read probe takes a multiple of 16 bytes")
+        self._run("probe", "lle_probe_read_stream", [_P, _L, _I, _P, _P], _ptr(data), nbytes, int(blocks), None)
+
+    def probe_mfma(self, dtype, blocks: int, iters: int) -> float:
+        """Launch a kernel of nothing but matrix instructions on registers; returns its flops."""
+        self._run("probe", "lle_probe_mfma", [_I, _I, _I, _P, _P], dtype_code(dtype), int(blocks), int(iters), None)
+        per_instruction = 2.0 * 16 * 16 * (32 if dtype == torch.bfloat16 else 4)
+        return per_instruction * 16 * iters * 4 * blocks
+
+
 _default: Optional[HipOps] = None
 
 
