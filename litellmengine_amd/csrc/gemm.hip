@@ -6,6 +6,7 @@
 // bfloat16 weight-streaming product of decoding, and its 32-bit twin (32-bit
 // operands through the 32-bit matrix instruction: products and sums in float32).
 #include "common.h"
+#include <type_traits>
 
 LLE_DEFINE_ERROR_STRING()
 
@@ -408,19 +409,21 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 // which may be lower: tile t of all workgroups together is one block of consecutive rows
 // (the memory channels see what they see of a plain sweep over W), of which workgroup b
 // takes the b-th piece.  The lanes of a tile that is not full read its last row again,
-// which costs no traffic.  A wavefront keeps two sets of W operands: while one is multiplied
-// the loads of the next are on their way, also across the end of a tile, where the
-// partial tiles are added up in LDS and written out.  X is read once per workgroup
-// instead of once per tile, and the sums of the folded norm are added up once.
+// which costs no traffic.  A wavefront keeps two sets of W operands (two steps each where
+// XS is even and small, one step otherwise): while one is multiplied the loads of the next are on
+// their way, also across the end of a tile, where the partial tiles are added up in LDS
+// and written out.  X is read once per workgroup instead of once per tile, and the sums of
+// the folded norm are added up once.
 // ---------------------------------------------------------------------------------
 template <bool GATED, bool SCALED, int XS, typename TC>
 __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X,
                                                                               const bf16_t* __restrict__ W,
                                                                               TC* __restrict__ C, int M, int N, int K,
                                                                               int share, NormFold fold) {
-    static_assert(XS % 4 == 0, "sets of two steps of W are multiplied in pairs");
     constexpr int WAVES = 16;
     constexpr int NT = GATED ? 2 : 1;
+    constexpr int SS = (XS % 2 == 0 && XS <= 6) ? 2 : 1;  // steps of a set (one where X takes most of the registers)
+    constexpr int SPT = XS / SS;             // sets of a tile
     __shared__ float s_acc[2][WAVES][NT][16][17];  // tiles take the two halves in turn: one barrier a tile
     __shared__ float s_inv[16];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
@@ -431,9 +434,9 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     auto tile_begin = [&](int t) { return (int)gridDim.x * 16 * t + (int)blockIdx.x * min(16, share - 16 * t); };
     auto tile_end = [&](int t) { return min(rows, tile_begin(t) + min(16, share - 16 * t)); };
 
-    // a set: two 64-element steps of the tile (and of the up tile that goes with a gate tile)
+    // a set: SS 64-element steps of the tile (and of the up tile that goes with a gate tile)
     struct Set {
-        gbf16x8 g0[2], g1[2], u0[2], u1[2];
+        gbf16x8 g0[SS], g1[SS], u0[SS], u1[SS];
     };
     // the load cursor: tile and step of the set that is asked for next
     int load_tile = 0, load_step = 0;
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     };
     auto load = [&](Set& set) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < SS; ++i) {
             const bf16_t* g = wp + (load_step + i) * (WAVES * SK_KSTEP);
             set.g0[i] = *(const gbf16x8*)g;
             set.g1[i] = *(const gbf16x8*)(g + 8);
@@ -455,16 +458,16 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
                 set.u1[i] = *(const gbf16x8*)(u + 8);
             }
         }
-        load_step += 2;
+        load_step += SS;
         if (load_step == XS) {
             load_step = 0;
             ++load_tile;
             aim();
         }
     };
-    Set a, b;
+    Set sets[2];
     aim();
-    load(a);
+    load(sets[0]);
     // rows of X beyond M are never written back, so their lanes may read any valid row
     gbf16x8 x0[XS], x1[XS];
     {
@@ -492,7 +495,7 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     gf32x4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const Set& set, int j) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < SS; ++i) {
             acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g0[i], x0[j + i], acc_g, 0, 0, 0);
             acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g1[i], x1[j + i], acc_g, 0, 0, 0);
             if (GATED) {
@@ -532,27 +535,37 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
         // which the threads that are still adding here have then passed.
         half ^= 1;
     };
-
-    int tile = 0;
-    for (; tile + 1 < tiles; ++tile) {  // every tile of the share but its last
+    // One tile: its sets in turn, the one after each asked for before it is multiplied (also the
+    // first of the next tile; the share's last tile asks for nothing beyond itself).  `first` is
+    // the buffer that holds the tile's first set: the sets alternate between the two buffers
+    // across tiles, so with an odd number of sets a tile every other tile starts in buffer 1.
+    auto run_tile = [&](int tile, auto first_c, bool last) {
+        constexpr int first = decltype(first_c)::value;
 #pragma unroll
-        for (int j = 0; j < XS; j += 4) {
-            load(b);
-            multiply(a, j);
-            load(a);  // after the tile's last set: the first of the next tile
-            multiply(b, j + 2);
+        for (int s = 0; s < SPT; ++s) {
+            if (!(last && s == SPT - 1)) load(sets[(first + s + 1) % 2]);
+            multiply(sets[(first + s) % 2], s * SS);
         }
         finish_tile(tile);
+    };
+    using Buf0 = std::integral_constant<int, 0>;
+    using Buf1 = std::integral_constant<int, 1>;
+    int tile = 0;
+    if constexpr (SPT % 2 == 0) {
+        for (; tile + 1 < tiles; ++tile) run_tile(tile, Buf0{}, false);
+        run_tile(tile, Buf0{}, true);
+    } else {
+        for (; tile + 2 < tiles; tile += 2) {
+            run_tile(tile, Buf0{}, false);
+            run_tile(tile + 1, Buf1{}, false);
+        }
+        if (tile + 1 < tiles) {
+            run_tile(tile, Buf0{}, false);
+            run_tile(tile + 1, Buf1{}, true);
+        } else {
+            run_tile(tile, Buf0{}, true);
+        }
     }
-    // the last one asks for nothing beyond itself
-#pragma unroll
-    for (int j = 0; j < XS; j += 4) {
-        load(b);
-        multiply(a, j);
-        if (j + 4 < XS) load(a);
-        multiply(b, j + 2);
-    }
-    finish_tile(tile);
 }
 
 // CUs of the current device (asked once per device)
@@ -568,20 +581,45 @@ static int gemm_compute_units() {
     return cached[dev];
 }
 
-// The streaming kernel takes the product when its shape is the one it is built for (K = 4096,
-// up to 16 rows) and W has more than one tile of rows for every CU.
+// The streaming kernel takes the product when K is a number of whole rounds of its 16 wavefronts
+// (1024 elements a round) that its registers hold, X has up to 16 rows, and W has more than one
+// tile of rows for every CU.
 template <bool GATED, bool SCALED, typename TC>
 static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K,
                                  const NormFold& fold, hipStream_t stream) {
-    constexpr int XS = 4;
-    if (M > 16 || K != SK_KSTEP * 16 * XS) return false;
+    if (M > 16 || K % (SK_KSTEP * 16) != 0) return false;
     const int rows = GATED ? N / 2 : N;
     const int units = gemm_compute_units();
     const int share = (rows + units - 1) / units;
     if (share <= 16) return false;
     const int blocks = (rows + share - 1) / share;
-    gemm_skinny_stream_kernel<GATED, SCALED, XS, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
-    return true;
+#define LLE_STREAM_CASE(XSV)                                                                                          \
+    case XSV:                                                                                                         \
+        gemm_skinny_stream_kernel<GATED, SCALED, XSV, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, \
+                                                                                               fold);                \
+        return true;
+    switch (K / (SK_KSTEP * 16)) {
+        LLE_STREAM_CASE(1)
+        LLE_STREAM_CASE(2)
+        LLE_STREAM_CASE(3)
+        LLE_STREAM_CASE(4)
+        LLE_STREAM_CASE(5)
+        case 6:
+        case 8:
+            if constexpr (!GATED) {  // the gated form's two tiles leave no registers for this much of X
+                if (K / (SK_KSTEP * 16) == 6) {
+                    gemm_skinny_stream_kernel<GATED, SCALED, 6, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K,
+                                                                                                          share, fold);
+                } else {
+                    gemm_skinny_stream_kernel<GATED, SCALED, 8, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K,
+                                                                                                          share, fold);
+                }
+                return true;
+            }
+            return false;
+    }
+#undef LLE_STREAM_CASE
+    return false;
 }
 
 template <typename TC, int NT, bool GATED>

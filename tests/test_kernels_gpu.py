@@ -147,6 +147,47 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         assert (got.double() - ref.double()).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("K", [1024, 2048, 3072, 4096, 5120, 6144, 8192])
+@pytest.mark.parametrize("M", [1, 7, 16])
+def test_streaming_products_at_every_width(M, K):
+    """The weight-streaming forms (one workgroup per CU walking over its share of W, X held in
+    registers) at every K they take, rows of W that leave the last tile of a share partly empty:
+    plain (both result types), gated, and both after a folded norm, against float64.  W is made
+    of rows that tell their own number, so a row written to the wrong place shows."""
+    from litellmengine_amd.parts import NormFold
+
+    o = ops()
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    N = 16 * units + 16 * 5 + 7  # more than one tile per CU, and no multiple of anything
+    x = rnd((M, K), torch.bfloat16, 51)
+    w = rnd((N, K), torch.bfloat16, 52, 0.05)
+    w[:, 0] = (torch.arange(N) % 64).to(torch.bfloat16) / 16  # tells the row
+    want = x.double() @ w.double().t()
+    lim = 2e-2 * max(1.0, want.abs().max().item())
+    for out_dtype in (torch.bfloat16, torch.float32):
+        got = o.linear(x, w, out_dtype)
+        assert (got.double() - want).abs().max() < (lim if out_dtype == torch.bfloat16 else lim / 100)
+    if K <= 5120:  # the gated form holds two tiles of W: it streams up to this width
+        half = N  # gate rows, then as many up rows
+        wg = torch.cat([w, rnd((half, K), torch.bfloat16, 53, 0.05)]).contiguous()
+        y = x.double() @ wg.double().t()
+        wantg = torch.nn.functional.silu(y[:, :half]) * y[:, half:]
+        got = o.gate_up_silu(x, wg)
+        assert got.shape == (M, half)
+        assert (got.double() - wantg).abs().max() < 2e-2 * max(1.0, wantg.abs().max().item())
+    # after a folded norm: the product before it makes the sums, this one applies the row factors
+    a = rnd((M, 64), torch.bfloat16, 54)
+    w1 = rnd((K, 64), torch.bfloat16, 55, 0.2)
+    hidden = rnd((M, K), torch.float32, 56, 1.5)
+    nw = (1 + 0.3 * rnd((K,), torch.float32, 57)).to(torch.bfloat16)
+    pre = o.linear(a, w1, fold=NormFold(hidden, nw, 1e-3))
+    h = hidden.double()
+    normed = h * torch.rsqrt((h ** 2).mean(1, keepdim=True) + 1e-3) * nw.double()
+    got = o.linear(pre, w)
+    wantn = normed @ w.double().t()
+    assert (got.double() - wantn).abs().max() < 2e-2 * max(1.0, wantn.abs().max().item())
+
+
 def test_silu_mul_reference_vector():
     # tests/test_silu_and_mul.cpp:48-56
     g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])
