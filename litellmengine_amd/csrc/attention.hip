@@ -1119,6 +1119,272 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     }
 }
 
+// ---------------------------------------------------------------------------------
+// float32 on the matrix cores: v_mfma_f32_16x16x4_f32 multiplies and adds float32 (no
+// reduced-precision mode), so this is still the true 32-bit path.  One kernel for every kind
+// of request, head sizes in steps of 16 up to 256, pages that hold a multiple of 16 keys:
+//   * a request with at most 16 rows (token, head of the group): one tile of rows, the four
+//     wavefronts take every fourth 16-key step and are merged through LDS (decoding);
+//   * any other: a workgroup takes 64 rows, each wavefront a tile of 16 of them and all keys
+//     that its rows see.
+// grid = (kv heads, row blocks x key splits, requests); with key splits the partial (m, l, acc)
+// go to the workspaces and the combine kernel merges them.
+// Operands (lane = (c, r), c = lane / 16, r = lane % 16): a lane loads 16 bytes, four
+// consecutive elements, and its element e is the contraction slot c of instruction e:
+//   S^T = K Q^T:    A = K[key r][16 q + 4 c + e],  B = Q[row r][16 q + 4 c + e]
+//   O^T += V^T P^T: A = V^T[element 16 n + r][key 4 c + e],  B = P[key 4 c + e][row r]
+// and the result tile S^T leaves lane (c, r) with keys 4 c .. 4 c + 3 of row r: exactly the B
+// operand of the second product, so P never leaves its registers.
+// ---------------------------------------------------------------------------------
+#define F32_WAVES 4
+#define F32_KEYS 16
+template <int DQ>
+__global__ __launch_bounds__(F32_WAVES* LLE_WAVE) void mfma_f32_attention_kernel(
+    const float* __restrict__ q, const float* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
+    const int32_t* __restrict__ kv_lens, float* __restrict__ out, float* __restrict__ ws_o,
+    float* __restrict__ ws_ml, int nsplit, int nq, int nkv, int P, int64_t page_stride, int max_pages, int window,
+    float scale_log2) {
+    constexpr int D = 16 * DQ;
+    extern __shared__ float smem[];  // [waves][16][D] acc, then [waves][16] m, [waves][16] l
+    float* s_o = smem;
+    float* s_m = smem + F32_WAVES * 16 * D;
+    float* s_l = s_m + F32_WAVES * 16;
+    const int s = blockIdx.z, kvh = blockIdx.x;
+    const int G = nq / nkv;
+    const int q_start = cu_tokens[s];
+    const int q_len = cu_tokens[s + 1] - q_start;
+    const int nrows = q_len * G;
+    if (nrows <= 0) return;
+    const int kv_len = kv_lens[s];
+    const int past = kv_len - q_len;
+    const int row_blocks = gridDim.y / nsplit;
+    const int split = blockIdx.y / row_blocks, yb = blockIdx.y % row_blocks;
+    const bool few = nrows <= 16;  // the same for the whole workgroup
+    const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
+    const int c = lane / 16, r16 = lane % 16;
+    if (few ? yb != 0 : yb * (16 * F32_WAVES) >= nrows) return;
+    const int row0 = few ? 0 : yb * (16 * F32_WAVES) + wave * 16;
+    const bool wave_has_rows = row0 < nrows;
+    const int32_t* table = block_tables + (int64_t)seq_slots[s] * max_pages;
+
+    // the lane's row
+    const int row = row0 + r16;
+    const bool exists = row < nrows;
+    const int tok = exists ? row / G : 0, g = exists ? row - tok * G : 0;
+    const int64_t head_row = (int64_t)(q_start + tok) * nq + kvh * G + g;
+    const int pos = exists ? past + tok : -1;
+    const int lo = (exists && window > 0) ? max(0, pos - window + 1) : 0;
+    f32x4 qf[DQ];
+#pragma unroll
+    for (int i = 0; i < DQ; ++i)
+        qf[i] = exists ? *(const f32x4*)(q + head_row * D + 16 * i + 4 * c) : f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // the keys of this wavefront's tile, in steps of 16, and its share of them
+    int step_begin = 0, step_end = 0, step_stride = 1;
+    if (wave_has_rows) {
+        const int last_row = min(nrows, row0 + 16) - 1;
+        const int hi = past + last_row / G;
+        const int lo_tile = window > 0 ? max(0, past + row0 / G - window + 1) : 0;
+        const int first = lo_tile / F32_KEYS, end = hi / F32_KEYS + 1;
+        const int per_split = (end - first + nsplit - 1) / nsplit;
+        step_begin = first + split * per_split;
+        step_end = min(end, step_begin + per_split);
+        if (few) {
+            step_begin += wave;
+            step_stride = F32_WAVES;
+        }
+    }
+    f32x4 o[DQ];
+#pragma unroll
+    for (int n = 0; n < DQ; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = NEG_BIG, l = 0.f;
+    const int64_t k_lane = ((int64_t)kvh * P + r16) * D + 4 * c;
+    const int64_t v_lane = ((int64_t)nkv + kvh) * P * D + (int64_t)r16 * P + 4 * c;
+    constexpr int NBUF = DQ <= 8 ? 2 : 1;
+    f32x4 kf[NBUF][DQ], vf[NBUF][DQ];
+    auto load = [&](int buf, int step) {
+        const int j0 = step * F32_KEYS;
+        const int lp = j0 / P, off = j0 - lp * P;  // 16 keys of a step lie in one page
+        const float* page = kv_layer + (int64_t)table[__builtin_amdgcn_readfirstlane(lp)] * page_stride;
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) kf[buf][i] = *(const f32x4*)(page + k_lane + (int64_t)off * D + 16 * i);
+#pragma unroll
+        for (int n = 0; n < DQ; ++n) vf[buf][n] = *(const f32x4*)(page + v_lane + (int64_t)16 * n * P + off);
+    };
+    auto multiply = [&](int buf, int step) {
+        const int j0 = step * F32_KEYS;
+        f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < DQ; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[buf][i][e], qf[i][e], sc, 0, 0, 0);
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int j = j0 + 4 * c + e;
+            x[e] = (j < lo || j > pos) ? NEG_BIG : sc[e] * scale_log2;
+        }
+        float top = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+        top = fmaxf(top, __shfl_xor(top, 16, LLE_WAVE));
+        top = fmaxf(top, __shfl_xor(top, 32, LLE_WAVE));
+        const float new_m = fmaxf(m, top);
+        // while the row has seen no key new_m is NEG_BIG as its masked scores are, and
+        // exp2(0) = 1 would count them: shift such rows so that they give 0
+        const float base = new_m <= NEG_BIG ? 0.f : new_m;
+        const float alpha = exp2f(m - base);
+        m = new_m;
+        f32x4 p;
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            p[e] = exp2f(x[e] - base);
+            psum += p[e];
+        }
+        l = l * alpha + psum;
+#pragma unroll
+        for (int n = 0; n < DQ; ++n) {
+            o[n] *= alpha;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[n] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[buf][n][e], p[e], o[n], 0, 0, 0);
+        }
+    };
+    if constexpr (NBUF == 2) {
+        // the operands of the next step are asked for before this one is multiplied
+        if (step_begin < step_end) load(0, step_begin);
+        int buf = 0;
+        for (int step = step_begin; step < step_end; step += step_stride) {
+            if (step + step_stride < step_end) {
+                if (buf == 0) load(1, step + step_stride); else load(0, step + step_stride);
+            }
+            if (buf == 0) multiply(0, step); else multiply(1, step);
+            buf ^= 1;
+        }
+    } else {  // heads over 128 elements: the registers hold one step's operands
+        for (int step = step_begin; step < step_end; step += step_stride) {
+            load(0, step);
+            multiply(0, step);
+        }
+    }
+    l += __shfl_xor(l, 16, LLE_WAVE);
+    l += __shfl_xor(l, 32, LLE_WAVE);
+
+    if (!few) {  // every wavefront writes the rows of its own tile
+        if (!exists) return;
+        if (nsplit > 1) {
+            float* po = ws_o + (head_row * nsplit + split) * D;
+#pragma unroll
+            for (int n = 0; n < DQ; ++n) *(f32x4*)(po + 16 * n + 4 * c) = o[n];
+            if (c == 0) {
+                ws_ml[(head_row * nsplit + split) * 2] = m;
+                ws_ml[(head_row * nsplit + split) * 2 + 1] = l;
+            }
+            return;
+        }
+        const float inv = 1.0f / l;
+#pragma unroll
+        for (int n = 0; n < DQ; ++n) *(f32x4*)(out + head_row * D + 16 * n + 4 * c) = o[n] * inv;
+        return;
+    }
+    // few rows: the four wavefronts hold parts of the same rows
+    if (exists) {
+#pragma unroll
+        for (int n = 0; n < DQ; ++n) *(f32x4*)(s_o + (wave * 16 + r16) * D + 16 * n + 4 * c) = o[n];
+    }
+    if (c == 0) {
+        s_m[wave * 16 + r16] = m;
+        s_l[wave * 16 + r16] = l;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
+        const int r = idx / D, e = idx - r * D;
+        float big = s_m[r];
+#pragma unroll
+        for (int w = 1; w < F32_WAVES; ++w) big = fmaxf(big, s_m[w * 16 + r]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < F32_WAVES; ++w) {
+            const float f = exp2f(s_m[w * 16 + r] - big);  // a wavefront without keys has l = 0, acc = 0
+            num += s_o[(w * 16 + r) * D + e] * f;
+            den += s_l[w * 16 + r] * f;
+        }
+        const int t = r / G, gg = r - t * G;
+        const int64_t hr = (int64_t)(q_start + t) * nq + kvh * G + gg;
+        if (nsplit == 1) {
+            out[hr * D + e] = num / den;
+        } else {
+            ws_o[(hr * nsplit + split) * D + e] = num;
+            if (e == 0) {
+                ws_ml[(hr * nsplit + split) * 2] = big;
+                ws_ml[(hr * nsplit + split) * 2 + 1] = den;
+            }
+        }
+    }
+}
+
+// merges the key splits of the kernel above: grid = (tokens, q heads), one wavefront each
+__global__ __launch_bounds__(LLE_WAVE) void f32_combine_kernel(const float* __restrict__ ws_o,
+                                                               const float* __restrict__ ws_ml, int nsplit,
+                                                               float* __restrict__ out, int nq, int D) {
+    const int64_t head_row = (int64_t)blockIdx.x * nq + blockIdx.y;
+    const int lane = threadIdx.x;
+    __shared__ float s_f[LLE_WAVE];
+    const float2 ml = *(const float2*)(ws_ml + (head_row * nsplit + min(lane, nsplit - 1)) * 2);
+    const float m = lane < nsplit ? ml.x : NEG_BIG, l = lane < nsplit ? ml.y : 0.f;
+    const float big = wave_max(m);
+    const float f = exp2f(m - big);
+    const float den = wave_sum(l * f);
+    s_f[lane] = f;
+    __syncthreads();
+    const float* o = ws_o + head_row * nsplit * D;
+    for (int e = lane; e < D; e += LLE_WAVE) {
+        float num = 0.f;
+        for (int k = 0; k < nsplit; ++k) num += o[(int64_t)k * D + e] * s_f[k];
+        out[head_row * D + e] = num / den;
+    }
+}
+
+// float32, head_dim a multiple of 16 (<= 256), page size a multiple of 16.  `row_blocks`: the
+// most 64-row blocks that a request of this batch has (1 when every request has at most 16
+// rows); with nsplit > 1 the workspaces ws_o [N * nq * nsplit * d] and ws_ml [N * nq * nsplit * 2]
+// floats are needed (nsplit <= 64).
+extern "C" int lle_paged_attention_mfma_f32(const void* q, const void* kv_layer, const void* block_tables,
+                                            const void* seq_slots, const void* cu_tokens, const void* kv_lens,
+                                            void* out, void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d,
+                                            int page_size, int64_t page_stride, int max_pages, int window,
+                                            float scale, int row_blocks, int nsplit, hipStream_t stream) {
+    if (N <= 0) return 0;
+    if (d % 16 != 0 || d > 256 || d <= 0 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
+    if (S > 65535 || nkv <= 0 || row_blocks < 1 || nsplit < 1 || nsplit > 64 || (int64_t)row_blocks * nsplit > 65535)
+        return (int)hipErrorInvalidValue;
+    if (nsplit > 1 && (!ws_o || !ws_ml)) return (int)hipErrorInvalidValue;
+    const float scale_log2 = scale * 1.44269504088896340736f;
+    const dim3 grid(nkv, row_blocks * nsplit, S);
+    const size_t smem = (size_t)(F32_WAVES * 16 * d + 2 * F32_WAVES * 16) * sizeof(float);
+#define LLE_F32_CASE(DQV)                                                                                        \
+    case DQV:                                                                                                    \
+        if (smem > 64 * 1024) {                                                                                  \
+            hipError_t e = hipFuncSetAttribute((const void*)mfma_f32_attention_kernel<DQV>,                       \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);           \
+            if (e != hipSuccess) return (int)e;                                                                  \
+        }                                                                                                        \
+        mfma_f32_attention_kernel<DQV><<<grid, F32_WAVES * LLE_WAVE, smem, stream>>>(                             \
+            (const float*)q, (const float*)kv_layer, (const int32_t*)block_tables, (const int32_t*)seq_slots,     \
+            (const int32_t*)cu_tokens, (const int32_t*)kv_lens, (float*)out, (float*)ws_o, (float*)ws_ml, nsplit, \
+            nq, nkv, page_size, page_stride, max_pages, window, scale_log2);                                      \
+        break;
+    switch (d / 16) {
+        LLE_F32_CASE(1) LLE_F32_CASE(2) LLE_F32_CASE(3) LLE_F32_CASE(4) LLE_F32_CASE(5) LLE_F32_CASE(6)
+        LLE_F32_CASE(7) LLE_F32_CASE(8) LLE_F32_CASE(9) LLE_F32_CASE(10) LLE_F32_CASE(11) LLE_F32_CASE(12)
+        LLE_F32_CASE(13) LLE_F32_CASE(14) LLE_F32_CASE(15) LLE_F32_CASE(16)
+    }
+#undef LLE_F32_CASE
+    if (nsplit > 1)
+        f32_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>((const float*)ws_o, (const float*)ws_ml, nsplit,
+                                                                 (float*)out, nq, d);
+    return (int)hipGetLastError();
+}
+
 // CUs of the current device (asked once per device)
 static int compute_units() {
     static int cached[64] = {0};

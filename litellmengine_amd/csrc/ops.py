@@ -291,6 +291,23 @@ class HipOps:
         win = int(window) if window else 0
         mfma = (q.dtype == torch.bfloat16 and d % 32 == 0 and page_size % 16 == 0 and max_q_len > 0
                 and max_kv_len > 0 and S <= 65535 and not self.force_generic_attention)
+        group = nq // nkv
+        if (q.dtype == torch.float32 and d % 16 == 0 and page_size % 16 == 0 and max_q_len > 0 and max_kv_len > 0
+                and S <= 65535 and not self.force_generic_attention):
+            # float32 on the matrix cores (float32 operands, products and sums)
+            rows = max_q_len * group
+            row_blocks = 1 if rows <= 16 else -(-rows // 64)
+            ns = self.f32_attention_splits(S, nkv, row_blocks, max_q_len, max_kv_len, win)
+            ws_o = ws_ml = None
+            if ns > 1:
+                ws_o = torch.empty((N * nq * ns * d,), dtype=torch.float32, device=q.device)
+                ws_ml = torch.empty((N * nq * ns * 2,), dtype=torch.float32, device=q.device)
+            self._run("attention", "lle_paged_attention_mfma_f32",
+                      [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _I, _P],
+                      _ptr(q), _ptr(kv_layer), _ptr(block_table), _ptr(seq_slots), _ptr(cu_tokens), _ptr(kv_lens),
+                      _ptr(out), _ptr(ws_o), _ptr(ws_ml), N, S, nq, nkv, d, page_size, kv_layer.stride(0),
+                      block_table.shape[1], win, float(scale), row_blocks, ns)
+            return out
         if not mfma:
             self._run("attention", "lle_paged_attention_generic",
                       [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _L, _I, _I, _F, _I, _P],
@@ -298,7 +315,6 @@ class HipOps:
                       _ptr(token_seq), _ptr(out), N, nq, nkv, d, page_size, kv_layer.stride(0), block_table.shape[1],
                       win, float(scale), dtype_code(q.dtype))
             return out
-        group = nq // nkv
         min_q_len = min_q_len or 1
         run_decode = min_q_len * group <= 16
         run_prefill = max_q_len * group > 16
@@ -421,6 +437,16 @@ class HipOps:
         if low <= resident or (tall <= resident and not window and 8 * past <= max_q_len):
             return 1
         return 2
+
+    def f32_attention_splits(self, num_seqs: int, num_kv_heads: int, row_blocks: int, max_q_len: int,
+                             max_kv_len: int, window: int) -> int:
+        """Key splits of the float32 matrix-core kernel: enough workgroups for the chip, at least
+        16 of its 16-key steps each."""
+        span = min(max_kv_len, window + max_q_len) if window else max_kv_len
+        steps = (span + 15) // 16
+        by_work = max(1, steps // 16)
+        by_fill = max(1, (2 * self.DECODE_TARGET_BLOCKS) // max(1, num_seqs * num_kv_heads * row_blocks))
+        return int(min(by_work, by_fill, 64))
 
     def decode_splits(self, num_seqs: int, num_kv_heads: int, max_kv_len: int, window: int) -> int:
         """Key splits of the decode kernel: enough workgroups to fill the chip, but

@@ -359,6 +359,42 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
     assert (got.double() - want.double()).abs().max() < tol(dtype, 2)
 
 
+@pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 16, 16, None), (16, 2, 64, 32, None),
+                                               (6, 1, 48, 16, 40), (2, 1, 256, 16, None), (32, 8, 128, 16, 700),
+                                               (3, 1, 160, 48, None), (5, 5, 80, 16, 9)])
+@pytest.mark.parametrize("lens", [
+    [(0, 9), (17, 1), (30, 2), (5, 11)],          # portions beside decoded tokens
+    [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
+    [(0, 150), (100, 70)],                        # prompt portions only, one after a past
+    [(2000, 49)],                                 # a short tail after a long past: keys split over workgroups
+    [(1500, 40), (1900, 1), (3, 30)],
+])
+def test_float32_matrix_core_attention(nq, nkv, d, P, window, lens):
+    """The float32 matrix-core kernel (float32 operands, products and sums) against the plain
+    form in float64 and against the generic kernel it stands beside."""
+    need = max((p + l + P - 1) // P for p, l in lens)
+    args, mq, mk = attention_case(torch.float32, nq, nkv, d, P, window, lens,
+                                  pages=sum((p + l + P - 1) // P for p, l in lens) + 3, max_pages=need + 1)
+    o = ops()
+    want = REF.paged_attention(*args).double()
+    got = o.paged_attention(*args, *mq, mk)
+    o.force_generic_attention = True
+    try:
+        generic = o.paged_attention(*args, *mq, mk)
+    finally:
+        o.force_generic_attention = False
+    assert (got.double() - want).abs().max() < tol(torch.float32, 2)
+    assert (generic.double() - want).abs().max() < tol(torch.float32, 2)
+    # one key made to stand out among all that a row sees: its value row comes back
+    q, kv, table, slots = args[0], args[1], args[2], args[3]
+    past, ql = lens[-1]
+    far = max(0, past + ql - 1 - (window - 1 if window else past + ql - 1))  # the first key the last row sees
+    page, off = int(table[int(slots[len(lens) - 1]), far // P]), far % P
+    kv[page, 0, 0, off, :] = q[-1, 0] * (60.0 / max(1.0, float((q[-1, 0] ** 2).sum()) ** 0.5))
+    got = o.paged_attention(*args, *mq, mk).reshape(-1, nq, d)
+    assert torch.allclose(got[-1, 0], v_pages(kv)[page, 0, :, off], atol=1e-3)
+
+
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 32, 16, None), (16, 2, 64, 32, None),
                                                (6, 1, 96, 16, 40), (8, 2, 256, 16, None), (32, 8, 128, 16, 700),
                                                (3, 1, 160, 48, None)])
