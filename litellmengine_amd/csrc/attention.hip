@@ -386,7 +386,7 @@ struct StepOperands {
 // this wavefront reads any key.  `after_first_loads()` runs once the first two steps are asked for.
 template <int DK, int RT, bool LOAD_Q = true, typename BeforeKeys, typename AfterFirstLoads>
 __device__ __forceinline__ void attend_rows(RowState<DK, RT>& st, const RowInfo (&row)[RT],
-                                            const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ table,
+                                            const bf16_t* kv_layer, const int32_t* __restrict__ table,
                                             int kvh, int nkv, int P, int64_t page_stride, int step_begin,
                                             int step_end, int step_stride, int lo_min, int hi, float scale_log2,
                                             BeforeKeys before_keys, AfterFirstLoads after_first_loads) {
@@ -657,7 +657,7 @@ __device__ __forceinline__ void fused_kv_write(const FusedQKV& f, int64_t tok, i
 #endif
 template <int DK, bool FUSED>
 __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
-    const bf16_t* __restrict__ q, bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
+    const bf16_t* __restrict__ q, bf16_t* kv_layer, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ seq_slots, const int32_t* __restrict__ cu_tokens,
     const int32_t* __restrict__ kv_lens, bf16_t* __restrict__ out, float* __restrict__ ws_o,
     float* __restrict__ ws_ml, int ws_stride, int nq, int nkv, int P, int64_t page_stride, int max_pages,
@@ -721,7 +721,11 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
                         if (step_of >= sb && step_of < se && (step_of - sb) % DEC_WAVES == wave)
                             fused_kv_write<DK>(fused, (int64_t)q_start + t, kvh, nq, nkv, kv_layer, P, page_stride);
                     }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    // The keys are read through the same pointer (no `restrict` on it: the pages are
+                    // written and read in this kernel), after this point in program order; the fence
+                    // keeps the compiler from moving those loads above the stores.
+                    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                    asm volatile("" ::: "memory");
                 }
             },
             [&]() { qrow.finish(st.qv[0], r16 < nrows, fused); });
