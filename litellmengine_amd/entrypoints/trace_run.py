@@ -37,27 +37,19 @@ def parse_args(argv=None):
     return p.parse_args(argv)
 
 
-def main(argv=None, stdin=None, stdout=None, ops=None, device=None) -> int:
-    args = parse_args(argv)
-    stdin = stdin or sys.stdin
-    stdout = stdout or sys.stdout
-    if args.max_tokens <= 0:
-        raise SystemExit("--max-tokens must be greater than 0")
-    if args.page_size <= 0:
-        raise SystemExit("--page-size must be positive")
-
+def replay(model, out_dir: str, max_tokens: int, page_size: int, max_requests: int, stdin, stdout) -> None:
+    """Feed the steps on `stdin` through `model` (a bound models.decoder.DecoderLM): one
+    ModelRunner.step per line, the wanted logits to `out_dir`, `done <step>` to `stdout`."""
     import numpy as np
     import torch
 
     from ..cache import CacheManager
     from ..engine import ModelRunner, StepEntry
-    from ..models import load_model
 
-    os.makedirs(args.out, exist_ok=True)
-    model = load_model(args.model, args.dtype, device=device, ops=ops)
-    num_pages = (args.max_tokens + args.page_size - 1) // args.page_size
+    os.makedirs(out_dir, exist_ok=True)
+    num_pages = (max_tokens + page_size - 1) // page_size
     cache = CacheManager(
-        model, page_size=args.page_size, num_pages=num_pages, max_requests=args.max_requests,
+        model, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
         dtype=model.ctx.dtype, device=model.ctx.device,
     )
     runner = ModelRunner(model, cache)
@@ -79,15 +71,28 @@ def main(argv=None, stdin=None, stdout=None, ops=None, device=None) -> int:
             logits = runner.step(entries)
             if logits.shape[0] > 0:
                 arr = logits.detach().to("cpu", torch.float32).contiguous().numpy().astype("<f4", copy=False)
-                tmp = os.path.join(args.out, f".{step}.f32.tmp")
+                tmp = os.path.join(out_dir, f".{step}.f32.tmp")
                 arr.tofile(tmp)
-                os.replace(tmp, os.path.join(args.out, f"{step}.f32"))
+                os.replace(tmp, os.path.join(out_dir, f"{step}.f32"))
         for rid in rec.get("end", []):
             rid = str(rid)
             if rid in slots:
                 runner.release(slots.pop(rid))
         stdout.write(f"done {step}\n")
         stdout.flush()
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    if args.max_tokens <= 0:
+        raise SystemExit("--max-tokens must be greater than 0")
+    if args.page_size <= 0:
+        raise SystemExit("--page-size must be positive")
+
+    from ..models import load_model
+
+    model = load_model(args.model, args.dtype)
+    replay(model, args.out, args.max_tokens, args.page_size, args.max_requests, sys.stdin, sys.stdout)
     return 0
 
 

@@ -140,15 +140,18 @@ def test_qwen3_8b_layer_sizes(tmp_path):
 def test_graph_replays_with_library_products(tmp_path):
     """Decode steps of 24 requests at the Qwen3-8B layer widths: more rows than the
     weight-streaming kernel takes, so the captured graph holds library matrix products.
-    Every replay is compared with the same step run without a graph."""
+    Every replay is compared with the same step run without a graph, and the rows of some
+    requests with the plain implementation's logits for their whole history."""
     from litellmengine_amd.config import Qwen3Config
-    from litellmengine_amd.models import random_model
+    from litellmengine_amd.weights import write_model_dir
 
     cfg = Qwen3Config.from_dict(dict(
         architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_size=4096, num_attention_heads=32,
         num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=32000, rope_theta=1e6,
         rms_norm_eps=1e-6, tie_word_embeddings=True))
-    model = random_model(cfg, seed=5, dtype="bfloat16")
+    d = str(tmp_path / "m24")
+    write_model_dir(cfg, d, 5, torch.bfloat16)
+    model = load_model(d, "bfloat16")
     B = 24
     prompts = [random_tokens(30 + 3 * i, cfg.vocab_size, 200 + i) for i in range(B)]
     feed = [random_tokens(8, cfg.vocab_size, 300 + i) for i in range(B)]
@@ -164,10 +167,14 @@ def test_graph_replays_with_library_products(tmp_path):
             got.append(runner.step([StepEntry(s, [feed[i][t]], [0]) for i, s in enumerate(slots)]).float().cpu())
             if t == 3:  # eager work between replays
                 extra = runner.admit() if cache.num_free_slots else None
-        outs[use_graphs] = torch.stack(got)
+        outs[use_graphs] = torch.stack(got)  # [step, request, vocabulary]
     diff = (outs[True] - outs[False]).abs().max().item()
     assert diff < 2e-2, diff
-    assert torch.isfinite(outs[True]).all()
+    pcfg, w = plain.read_model_dir(d, dtype=torch.float32)
+    for i in (0, 11, 23):
+        want = plain.model_logits_fast(prompts[i] + feed[i], w, pcfg)[len(prompts[i]):].double()
+        err = (outs[True][:, i].double() - want).abs().max().item() / max(1.0, want.abs().max().item())
+        assert err < 4e-2, (i, err)
 
 
 ODD = [

@@ -208,9 +208,8 @@ def test_greedy_generation_through_the_entry_point(tmp_path, which, dtype):
     got = generate(d, prompts, max_tokens=8, temperature=0.0, dtype=dtype, page_size=4, prefill_chunk=16)
     if dtype == "float32":
         assert got == want
-    else:  # rounding may flip a near-tie; after a flip the sequences part ways
-        first = [next((i for i, (a, b) in enumerate(zip(g, x)) if a != b), 8) for g, x in zip(got, want)]
-        assert sum(first) >= 24, (got, want)
+    else:  # rounding may flip a near-tie, after which the sequences part ways: near the maximum at every step
+        assert all(len(g) == 8 and near_greedy(p, g, w, cfg, 8e-2) for p, g in zip(prompts, got)), (got, want)
 
 
 @pytest.mark.gpu

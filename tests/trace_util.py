@@ -111,16 +111,20 @@ def run_tool(model_dir: str, dtype: str, out_dir: str, trace: TraceBuilder, max_
              page_size: int = None, in_process_ops=None) -> None:
     """Run bin/trace_run over the trace (as a child process, as a user would;
     `in_process_ops` runs its main() here on the CPU with substitute kernels)."""
-    argv = ["--model", model_dir, "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens or trace.max_tokens)]
-    if page_size:
-        argv += ["--page-size", str(page_size)]
+    max_tokens = max_tokens or trace.max_tokens
     if in_process_ops is not None:
-        from litellmengine_amd.entrypoints.trace_run import main
+        # the tool's own loop over the steps, with a model loaded here for the CPU stand-in kernels
+        from litellmengine_amd.entrypoints.trace_run import replay
+        from litellmengine_amd.models import load_model
 
         out = io.StringIO()
-        assert main(argv, stdin=io.StringIO(trace.text()), stdout=out, ops=in_process_ops, device="cpu") == 0
+        model = load_model(model_dir, dtype, device="cpu", ops=in_process_ops)
+        replay(model, out_dir, max_tokens, page_size or 16, 16, io.StringIO(trace.text()), out)
         done = out.getvalue().split("\n")
     else:
+        argv = ["--model", model_dir, "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens)]
+        if page_size:
+            argv += ["--page-size", str(page_size)]
         proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run")] + argv, input=trace.text(),
                               text=True, capture_output=True, timeout=600)
         assert proc.returncode == 0, proc.stderr[-3000:]
