@@ -409,23 +409,29 @@ def test_chat_template_belongs_to_the_architecture(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_shrinking_batch_walks_through_few_graphs(tmp_path, dtype):
+@pytest.mark.parametrize("dtype,max_graphs", [("float32", 32), ("bfloat16", 32), ("float32", 2)])
+def test_a_shrinking_batch_walks_through_few_graphs(tmp_path, dtype, max_graphs):
     """Thirteen requests that finish one after the other: the decode batch shrinks from 13 to 1,
     padded to 16, 8, 4, 2, 1 with rows that stand for nobody, so five graphs are captured, not
-    thirteen; every request generates what the plain model generates."""
+    thirteen; every request generates what the plain model generates.  A second wave finds the
+    graphs again, unless only two may be kept: then the ones used least recently were dropped
+    and are captured anew."""
     d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
     cfg, w = plain.read_model_dir(d)
     model = load_model(d, dtype)
     eng = LLMEngine(model, page_size=16, num_pages=13 * 4, max_requests=13, max_tokens_per_step=512)
-    prompts = [random_tokens(5 + 2 * i, 419, 300 + i) for i in range(13)]
-    reqs = [eng.add_request(p, 2 + i) for i, p in enumerate(prompts)]  # the i-th finishes after 2 + i tokens
-    eng.run_until_finished()
-    assert eng.runner.use_graphs and eng.runner.num_captures <= 5, eng.runner.num_captures
-    assert sorted(k[0] for k in eng.runner._graphs) == [1, 2, 4, 8, 16]
-    for r, p in zip(reqs, prompts):
-        if dtype == "float32":
-            assert r.generated == plain.generate_greedy(p, w, cfg, r.max_new_tokens)
-        else:
-            assert len(r.generated) == r.max_new_tokens and near_greedy(p, r.generated, w, cfg, 8e-2)
-    assert all(g.pool.num_held == 0 for g in eng.cache.groups)
+    eng.runner.MAX_GRAPHS = max_graphs
+    for wave in range(2):
+        prompts = [random_tokens(5 + 2 * i, 419, 300 + 20 * wave + i) for i in range(13)]
+        reqs = [eng.add_request(p, 2 + i) for i, p in enumerate(prompts)]  # the i-th finishes after 2 + i tokens
+        eng.run_until_finished()
+        assert eng.runner.use_graphs and len(eng.runner._graphs) <= max_graphs
+        assert eng.runner.num_captures == (5 if max_graphs >= 5 else 5 * (wave + 1)), eng.runner.num_captures
+        if max_graphs >= 5:
+            assert sorted(k[0] for k in eng.runner._graphs) == [1, 2, 4, 8, 16]
+        for r, p in zip(reqs, prompts):
+            if dtype == "float32":
+                assert r.generated == plain.generate_greedy(p, w, cfg, r.max_new_tokens)
+            else:
+                assert len(r.generated) == r.max_new_tokens and near_greedy(p, r.generated, w, cfg, 8e-2)
+        assert all(g.pool.num_held == 0 for g in eng.cache.groups)
