@@ -3,6 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
+    python bench.py --dtype float32                               # the same in true 32-bit
+    python bench.py --sizes 32b | --sizes 0p6b                    # the decode workload at other layer sizes
     python bench.py --workload reference-0p6b [--dtype float32]   # the reference's own benchmark shape
     python bench.py --workload mixed-32b [--layers L]             # a prompt chunk beside 63 decoded tokens
 
@@ -12,7 +14,9 @@ paged cache, sampling) with `batch` live requests whose context ends at
 One JSON line is printed: `value` = decoded tokens per second, `prefill` = a
 2048-token prompt in one step, `roofline` = bytes the decode step has to read
 (every weight it uses once + the cache of the live requests) / its time against
-8 TB/s, `points` = decode at batch 1 and 64.  The reference publishes nothing
+8 TB/s, `points` = decode at batch 1 and 64.  Both rooflines are also given against
+what this machine reaches on kernels that do nothing else (`measured_peak`: a
+read-only kernel over 4 GiB, a kernel of matrix instructions on registers).  The reference publishes nothing
 for this configuration (its only table is Qwen3-0.6B in float32 on an unnamed
 GPU, readme.md:62-66), so `vs_baseline` is null.
 """
@@ -284,6 +288,8 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b"],
+                    help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B")
     ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
                          "sizes, or a mixed prompt-portion + decode step at Qwen3-32B sizes")
@@ -306,8 +312,11 @@ def main():
     from litellmengine_amd.config import Qwen3Config
     from litellmengine_amd.models import random_model
 
-    sizes = dict(SIZES, num_hidden_layers=args.layers)
+    table = {"8b": SIZES, "0p6b": SIZES_0P6B, "32b": SIZES_32B}[args.sizes]
+    layers = args.layers if args.layers != SIZES["num_hidden_layers"] or args.sizes == "8b" else table["num_hidden_layers"]
+    sizes = dict(table, num_hidden_layers=layers)
     cfg = Qwen3Config.from_dict(sizes)
+    name = {"8b": "Qwen3-8B", "0p6b": "Qwen3-0.6B", "32b": "Qwen3-32B"}[args.sizes]
     torch.cuda.set_device(0)
     model = random_model(cfg, seed=0, dtype=args.dtype)
     elem = 2 if args.dtype == "bfloat16" else 4
@@ -319,7 +328,7 @@ def main():
     step_bytes = weight_bytes_per_step(cfg, elem) + args.batch * avg_ctx * kv_bytes_per_token(cfg, elem)
     achieved = step_bytes / dt
     line = {
-        "metric": "decode tok/s @ batch 8, Qwen3-8B sizes, context 4096 (+ prefill tok/s @ 2048, % roofline)",
+        "metric": f"decode tok/s @ batch {args.batch}, {name} sizes, context {args.context} (+ prefill tok/s @ 2048, % roofline)",
         "value": round(value, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -332,8 +341,8 @@ def main():
         "dtype": short,
         "data": "synthetic: seeded random weights, uniform random token ids",
         "config": {
-            "model": "Qwen3-8B sizes (random weights)", "layers": cfg.num_hidden_layers,
-            "layers_of_full_model": SIZES["num_hidden_layers"], "hidden": cfg.hidden_size,
+            "model": f"{name} sizes (random weights)", "layers": cfg.num_hidden_layers,
+            "layers_of_full_model": table["num_hidden_layers"], "hidden": cfg.hidden_size,
             "q_heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "global_batch": args.batch,
             "seq_len": args.context, "page_size": PAGE_SIZE, "prefill_tokens": PREFILL_TOKENS, "parallelism": "none (1 GPU)",

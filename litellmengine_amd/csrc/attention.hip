@@ -699,6 +699,10 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
     const int se = min(last + 1, sb + per_split);
     // keys of later splits are not this workgroup's: attend_rows may run a step past `se`
     row[0].pos = min(row[0].pos, se * KSTEP - 1);
+    // ... and asks for operands two steps ahead: past this split's last key those loads go to the
+    // split's own last page (which the caches hold) instead of the next split's pages, which would
+    // travel from memory twice, once for each of the two workgroups
+    const int hi_loads = max(lo_min, min(hi, se * KSTEP - 1));
 
     RowState<DK, 1> st;
     if constexpr (FUSED) {
@@ -712,7 +716,7 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
         const int rr = r16 < nrows ? r16 : 0;
         const int64_t tok = (int64_t)q_start + rr / G;
         attend_rows<DK, 1, false>(
-            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi, scale_log2,
+            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi_loads, scale_log2,
             [&]() {
                 qrow.load(fused.qkv + (tok * (nq + 2 * nkv) + kvh * G + rr % G) * D, fused, tok);
                 if (fused.write_kv) {
@@ -731,7 +735,7 @@ __global__ __launch_bounds__(DEC_WAVES* LLE_WAVE) void mfma_decode_kernel(
             [&]() { qrow.finish(st.qv[0], r16 < nrows, fused); });
     } else {
         attend_rows<DK, 1, true>(
-            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi, scale_log2,
+            st, row, kv_layer, table, kvh, nkv, P, page_stride, sb + wave, se, DEC_WAVES, lo_min, hi_loads, scale_log2,
             []() {}, []() {});
     }
 
