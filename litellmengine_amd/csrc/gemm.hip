@@ -200,8 +200,12 @@ template <int MT, int NT, bool GATED, bool RESID, bool SCALED, typename TC, int 
 __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                          const bf16_t* __restrict__ W,
                                                                          TC* __restrict__ C, int M, int N, int K,
-                                                                         NormFold fold) {
+                                                                         int tile_rows, NormFold fold) {
     static_assert(!(RESID || SCALED) || MT <= 2, "the norm is folded for up to 32 rows");
+    // `tile_rows` (at most 16) rows of W per tile: fewer than 16 where that makes the number of tiles a
+    // multiple of the number of CUs (see skinny_tile_rows); the lanes past them read the tile's last
+    // row again, which costs no traffic, and write nothing.  Forms with several tiles of W per
+    // workgroup (NT > 1, not gated) keep whole tiles.
     // NT tiles of 16 rows of W per workgroup share the X operands they are multiplied with
     __shared__ float s_acc[SK_WAVES][NT][MT][16][17];
     __shared__ float s_inv[16 * MT];
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
     // trip of its own), and the small loads beside W (parts of the norm's sums, residual
     // stream, norm weight) are asked for without a condition around them, so that nothing
     // waits for them before the loads of W are on their way.
-    asm volatile("" ::"s"(X), "s"(W), "s"(C), "s"(M), "s"(N), "s"(K), "s"(fold.hidden), "s"(fold.weight),
+    asm volatile("" ::"s"(X), "s"(W), "s"(C), "s"(M), "s"(N), "s"(K), "s"(tile_rows), "s"(fold.hidden), "s"(fold.weight),
                  "s"(fold.weight_dtype), "s"(fold.xw), "s"(fold.ss_out), "s"(fold.ss_in), "s"(fold.parts),
                  "s"(fold.eps));
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
@@ -225,7 +229,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
             early[i] = fold.ss_in[(int64_t)wave * fold.parts + min(lane + LLE_WAVE * i, fold.parts - 1)];
     }
     const int c = lane / 16, r16 = lane % 16;
-    const int64_t n0 = (int64_t)blockIdx.x * (GATED ? 16 : 16 * NT);
+    const int64_t n0 = (int64_t)blockIdx.x * ((GATED || NT == 1) ? tile_rows : 16 * NT);
     // RESID: thread (m, n) of the first 256 owns element [m][n0 + n]; what it needs of the
     // residual stream and of the norm weight is asked for now and has arrived by the epilogue
     // (all threads ask, for places that are there; the bits of the weight are read as they lie
@@ -235,7 +239,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) resid_h[mt] = 0.f;
     if (RESID) {
-        const int64_t col = min(n0 + threadIdx.x % 16, (int64_t)N - 1);
+        const int64_t col = min(n0 + min((int)(threadIdx.x % 16), tile_rows - 1), (int64_t)N - 1);
         if (fold.weight_dtype == LLE_F32)
             resid_w = ((const uint32_t*)fold.weight)[col];
         else
@@ -247,8 +251,9 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
     const bf16_t* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int64_t wrow = GATED ? min(n0 + r16, (int64_t)N / 2 - 1) + nt * ((int64_t)N / 2)
-                                   : min(n0 + 16 * nt + r16, (int64_t)N - 1);
+        const int rt = min(r16, tile_rows - 1);  // the lane's row of the tile
+        const int64_t wrow = GATED ? min(n0 + rt, (int64_t)N / 2 - 1) + nt * ((int64_t)N / 2)
+                                   : min(n0 + (NT == 1 ? rt : 16 * nt + r16), (int64_t)N - 1);
         wp[nt] = W + wrow * K + 16 * c;
     }
     // rows of X beyond M are never written back, so their lanes may read any valid row
@@ -347,7 +352,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
         for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
             const int mt = idx / 256, m = (idx / 16) % 16, n = idx % 16;
             const int64_t row = 16 * mt + m, col = n0 + n;
-            if (row >= M || col >= N / 2) continue;
+            if (row >= M || col >= N / 2 || n >= tile_rows) continue;
             float g = 0.f, u = 0.f;
 #pragma unroll
             for (int w = 0; w < SK_WAVES; ++w) {
@@ -370,7 +375,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
             for (int mt = 0; mt < MT; ++mt) {
                 const int m16 = threadIdx.x / 16, m = 16 * mt + m16;
                 float sq = 0.f;
-                if (m < M && col < N) {
+                if (m < M && col < N && n < tile_rows) {
                     float sum = 0.f;
 #pragma unroll
                     for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][0][mt][n][m16];
@@ -390,7 +395,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
     for (int idx = threadIdx.x; idx < NT * MT * 256; idx += blockDim.x) {
         const int nt = idx / (MT * 256), mt = (idx / 256) % MT, m = (idx / 16) % 16, n = idx % 16;
         const int64_t row = 16 * mt + m, col = n0 + 16 * nt + n;
-        if (row >= M || col >= N) continue;
+        if (row >= M || col >= N || (NT == 1 && n >= tile_rows)) continue;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][nt][mt][n][m];
@@ -622,19 +627,40 @@ static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M,
     return false;
 }
 
+// Rows of W per tile of the one-tile-per-workgroup kernel.  16 (a whole matrix-core tile) while the
+// tiles are at most one per CU or fill whole rounds of the CUs; otherwise as many as make the last
+// round full: with 320 tiles of 16 rows on 256 CUs a quarter of the CUs reads twice what the others
+// read and the launch lasts as long as two rounds, with 512 tiles of 10 rows every CU reads the same.
+static int skinny_tile_rows(int rows) {
+    const int units = gemm_compute_units();
+    const int tiles16 = (rows + 15) / 16;
+    if (tiles16 <= units) return 16;
+    const int rounds = (tiles16 + units - 1) / units;
+    const int per_tile = (int)(((int64_t)rows + (int64_t)rounds * units - 1) / ((int64_t)rounds * units));
+    return per_tile < 1 ? 1 : (per_tile > 16 ? 16 : per_tile);
+}
+
+// tiles of lle_gemm_skinny_resid_bf16 for a weight of N rows: the second size of its ss_part
+extern "C" int lle_gemm_skinny_resid_parts(int N) {
+    if (N <= 0) return 0;
+    const int tr = skinny_tile_rows(N);
+    return (N + tr - 1) / tr;
+}
+
 template <typename TC, int NT, bool GATED>
 static int launch_skinny(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K, hipStream_t stream) {
     constexpr int WAVES = 16, UNROLL = 4 / NT;
     const int rows = GATED ? N / 2 : N;
-    const int per_block = GATED ? 16 : 16 * NT;
+    const int tile_rows = (GATED || NT == 1) ? skinny_tile_rows(rows) : 16;
+    const int per_block = (GATED || NT == 1) ? tile_rows : 16 * NT;
     const int blocks = (rows + per_block - 1) / per_block;
     const int mt = (M + 15) / 16;
     const NormFold none = {};
     switch (mt) {
-        case 1: gemm_skinny_kernel<1, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
-        case 2: gemm_skinny_kernel<2, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
-        case 3: gemm_skinny_kernel<3, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
-        case 4: gemm_skinny_kernel<4, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, none); break;
+        case 1: gemm_skinny_kernel<1, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, tile_rows, none); break;
+        case 2: gemm_skinny_kernel<2, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, tile_rows, none); break;
+        case 3: gemm_skinny_kernel<3, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, tile_rows, none); break;
+        case 4: gemm_skinny_kernel<4, NT, GATED, false, false, TC, WAVES, UNROLL><<<blocks, WAVES * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, tile_rows, none); break;
         default: return (int)hipErrorInvalidValue;
     }
     return (int)hipGetLastError();
@@ -673,8 +699,8 @@ extern "C" int lle_gemm_skinny_gated_bf16(const void* X, const void* W, void* C,
 
 // The product BEFORE a folded norm: delta = X W^T [M, N] is added into `hidden` (float32 [M, N],
 // in place), xw = hidden * norm_weight goes to `xw` (bfloat16 [M, N]) and the sums of squares of
-// the new hidden over each workgroup's 16 columns to ss_part [16 or 32][(N + 15) / 16] (32 rows
-// when M > 16).  1 <= M <= 32.
+// the new hidden over each workgroup's columns to ss_part [16 or 32][lle_gemm_skinny_resid_parts(N)]
+// (32 rows when M > 16).  1 <= M <= 32.
 extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hidden, const void* norm_weight,
                                           int weight_dtype, void* xw, void* ss_part, int M, int N, int K,
                                           hipStream_t stream) {
@@ -686,12 +712,13 @@ extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hi
     fold.weight_dtype = weight_dtype;
     fold.xw = (bf16_t*)xw;
     fold.ss_out = (float*)ss_part;
+    const int tr = skinny_tile_rows(N), blocks = (N + tr - 1) / tr;
     if (M <= 16)
-        gemm_skinny_kernel<1, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
-            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
+        gemm_skinny_kernel<1, 1, false, true, false, bf16_t, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, tr, fold);
     else
-        gemm_skinny_kernel<2, 1, false, true, false, bf16_t, 16, 4><<<(N + 15) / 16, 16 * LLE_WAVE, 0, stream>>>(
-            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, fold);
+        gemm_skinny_kernel<2, 1, false, true, false, bf16_t, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(
+            (const bf16_t*)X, (const bf16_t*)W, (bf16_t*)nullptr, M, N, K, tr, fold);
     LLE_RETURN_LAUNCH_STATUS();
 }
 
@@ -713,14 +740,18 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     const int threads = 16 * LLE_WAVE;
     if (gated && launch_skinny_stream<true, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
     } else if (!gated && launch_skinny_stream<false, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
-    } else if (gated && M <= 16)
-        gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
-    else if (gated)
-        gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<(N / 2 + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
-    else if (M <= 16)
-        gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
-    else
-        gemm_skinny_kernel<2, 1, false, false, true, bf16_t, 16, 4><<<(N + 15) / 16, threads, 0, stream>>>(x, w, c, M, N, K, fold);
+    } else {
+        const int rows = gated ? N / 2 : N;
+        const int tr = skinny_tile_rows(rows), blocks = (rows + tr - 1) / tr;
+        if (gated && M <= 16)
+            gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+        else if (gated)
+            gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+        else if (M <= 16)
+            gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+        else
+            gemm_skinny_kernel<2, 1, false, false, true, bf16_t, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+    }
     LLE_RETURN_LAUNCH_STATUS();
 }
 

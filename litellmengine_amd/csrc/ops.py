@@ -130,6 +130,13 @@ class HipOps:
         most = 32 if width <= self.SKINNY_SMALL_WIDTH else self.SKINNY_MAX_ROWS
         return dtype == torch.bfloat16 and 0 < rows <= most and width % 8 == 0 and not self.force_library_gemm
 
+    def norm_sum_parts(self, width: int) -> int:
+        """Into how many column ranges the product before a folded norm over `width` splits the
+        sums of squares (one per tile of its launch; the kernel library decides the tiles)."""
+        fn = getattr(build.load_library("gemm"), "lle_gemm_skinny_resid_parts")
+        fn.argtypes, fn.restype = [_I], _I
+        return int(fn(int(width)))
+
     def _linear_folded(self, x, weight, fold, gated: bool):
         """The forms of the weight-streaming product around a folded norm: `x` a Prenormed
         (its row factors are applied to the result), `fold` a NormFold (the result goes
@@ -160,7 +167,7 @@ class HipOps:
               f"residual stream {list(fold.hidden.shape)} does not fit a product [{M}, {N}]")
         _need(self.can_fold_norm(M, N, xin.dtype), f"a norm over {N} cannot be folded for {M} rows")
         xw = torch.empty((M, N), dtype=torch.bfloat16, device=xin.device)
-        sums = torch.empty((16 if M <= 16 else 32, (N + 15) // 16), dtype=torch.float32, device=xin.device)
+        sums = torch.empty((16 if M <= 16 else 32, self.norm_sum_parts(N)), dtype=torch.float32, device=xin.device)
         self._run("gemm", "lle_gemm_skinny_resid_bf16", [_P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
                   _ptr(xin), _ptr(weight), _ptr(fold.hidden), _ptr(fold.weight), dtype_code(fold.weight.dtype),
                   _ptr(xw), _ptr(sums), M, N, K)

@@ -87,7 +87,7 @@ def test_silu_mul(dtype, I):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,I,K", [(1, 128, 64), (5, 200, 96), (8, 12288, 4096), (8, 136, 80), (9, 100, 72), (40, 64, 48),
-                                   (3, 12277, 4096), (1, 8189, 4096)])
+                                   (3, 12277, 4096), (1, 8189, 4096), (7, 4500, 200), (16, 5003, 72)])
 def test_gate_up_silu(dtype, M, I, K):
     x = rnd((M, K), dtype, 21, 2.0)
     w = rnd((2 * I, K), dtype, 22, 0.1)
@@ -103,7 +103,9 @@ def test_gate_up_silu(dtype, M, I, K):
 @pytest.mark.parametrize("M,H,K,N", [(1, 64, 40, 48), (3, 136, 72, 100), (8, 4096, 1024, 512), (5, 1000, 64, 30),
                                      (6, 4096, 256, 8189), (1, 4096, 128, 12288), (16, 4096, 256, 6151), (11, 5120, 128, 260),
                                      (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70), (32, 1024, 2048, 3072),
-                                     (17, 72, 40, 22), (29, 2048, 512, 128)])
+                                     (17, 72, 40, 22), (29, 2048, 512, 128),
+                                     # more tiles than CUs, no whole rounds: tiles of fewer than 16 rows
+                                     (9, 4600, 64, 4700), (16, 5120, 128, 5000), (3, 6152, 40, 4099)])
 def test_norm_folded_into_products(wdtype, M, H, K, N):
     """RMSNorm between two products, done by them: the first adds its result into the
     residual stream and leaves hidden * w and sums of squares, the second (plain or
@@ -127,7 +129,7 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         pre = o.linear(a, w1, fold=NormFold(h, nw, eps))
         want_h = hidden.double() + a.double() @ w1.double().t()
         assert (h.double() - want_h).abs().max() < 1e-4 * max(1.0, want_h.abs().max().item())
-        assert pre.sums.shape == (16 if M <= 16 else 32, (H + 15) // 16)
+        assert pre.sums.shape == (16 if M <= 16 else 32, o.norm_sum_parts(H)) and o.norm_sum_parts(H) >= (H + 15) // 16
         ss = pre.sums.double().sum(1)[:M]
         assert torch.allclose(ss, (want_h ** 2).sum(1), rtol=1e-5)
         normed = want_h * torch.rsqrt((want_h ** 2).mean(1, keepdim=True) + eps) * nw.double()
@@ -201,7 +203,8 @@ def test_silu_mul_reference_vector():
                                                 (torch.bfloat16, torch.bfloat16)])
 @pytest.mark.parametrize("M,N,K", [(1, 503, 96), (2, 4, 3), (5, 130, 70), (67, 257, 200), (33, 1000, 4096),
                                    (8, 6144, 4096), (16, 311, 136), (17, 48, 64), (64, 4096, 1536), (49, 72, 40),
-                                   (3, 151936, 128), (5, 8189, 4096), (2, 6151, 4096), (16, 4112, 4096)])
+                                   (3, 151936, 128), (5, 8189, 4096), (2, 6151, 4096), (16, 4112, 4096),
+                                   (5, 5120, 1600), (16, 4200, 72), (9, 4603, 25600)])
 def test_linear(in_dtype, out_dtype, M, N, K):
     x = rnd((M, K), in_dtype, 6)
     w = rnd((N, K), in_dtype, 7, 0.05)
