@@ -30,6 +30,7 @@
 //    share the K/V tiles through LDS, two workgroups share a CU.
 #include "common.h"
 #include <type_traits>
+#include <mutex>
 
 LLE_DEFINE_ERROR_STRING()
 
@@ -1424,6 +1425,31 @@ static int launch_decode(const bf16_t* q, bf16_t* kv_layer, const int32_t* block
     return 0;
 }
 
+// A second stream of this library's own (per device, made at first use, default priority) and the
+// two events that fork it from and join it to the caller's stream: in a batch that holds prompt
+// portions beside decoded tokens the two attention kernels work on different requests, one bound by
+// memory and one by the matrix cores, and share the chip instead of taking turns.
+struct SideLane {
+    hipStream_t stream;
+    hipEvent_t fork, join;
+};
+static SideLane* side_lane() {
+    static SideLane lanes[64];
+    static int state[64] = {0};  // 0: not made, 1: there, -1: could not be made
+    static std::mutex lock;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> guard(lock);
+    if (state[dev] == 0) {
+        SideLane& l = lanes[dev];
+        const bool ok = hipStreamCreateWithFlags(&l.stream, hipStreamNonBlocking) == hipSuccess &&
+                        hipEventCreateWithFlags(&l.fork, hipEventDisableTiming) == hipSuccess &&
+                        hipEventCreateWithFlags(&l.join, hipEventDisableTiming) == hipSuccess;
+        state[dev] = ok ? 1 : -1;
+    }
+    return state[dev] == 1 ? &lanes[dev] : nullptr;
+}
+
 template <int DK>
 static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_tables,
                        const int32_t* seq_slots, const int32_t* cu_tokens, const int32_t* kv_lens,
@@ -1437,6 +1463,14 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
     if (!run_prefill) nsplit_prefill = 1;
     const int ws_stride = nsplit_decode > nsplit_prefill ? nsplit_decode : nsplit_prefill;
     if (fused.qkv && (run_prefill || !run_decode || DK % 2 != 0)) return (int)hipErrorInvalidValue;
+    // both kinds in one batch: the decode kernel goes to the side stream, forked from and joined to `stream`
+    SideLane* lane = (run_decode && run_prefill) ? side_lane() : nullptr;
+    hipStream_t prefill_stream = stream;
+    if (lane) {
+        if (hipEventRecord(lane->fork, stream) != hipSuccess || hipStreamWaitEvent(lane->stream, lane->fork, 0) != hipSuccess)
+            lane = nullptr;
+    }
+    if (lane) stream = lane->stream;  // for the decode kernel below
     if (run_decode) {
         int e;
         if constexpr (DK % 2 == 0) {
@@ -1452,6 +1486,10 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
                                          nsplit_decode, fused, stream);
         }
         if (e != 0) return e;
+    }
+    if (lane) {
+        if (hipEventRecord(lane->join, lane->stream) != hipSuccess) return (int)hipGetLastError();
+        stream = prefill_stream;
     }
     if (run_prefill) {
         const int rows = max_q_len * G;
@@ -1469,6 +1507,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
         else
             launch(std::integral_constant<int, PRE_RT_OF(DK)>{});
     }
+    if (lane && hipStreamWaitEvent(stream, lane->join, 0) != hipSuccess) return (int)hipGetLastError();
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
         mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(
             ws_o, ws_ml, ws_stride, cu_tokens, token_seq, out, nq, nkv, D, run_decode ? nsplit_decode : nsplit_prefill,
