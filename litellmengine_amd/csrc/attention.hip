@@ -196,6 +196,21 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define LAZY_MAX 8.0f  // a row's reference maximum may lag its true one by this much (base 2)
 #define KSTEP 32  // keys per step: two 16-key tiles; pages hold a multiple of 16 keys
 #define KEY_OF_ROW(r, x) (8 * ((r) / 4) + 4 * (x) + (r) % 4)
+// LDS tiles of the prompt kernel.  LDS has 64 banks of 4 bytes; a 16-byte read of a wavefront
+// is served sixteen lanes a cycle, and the sixteen are not consecutive (measured: a cycle takes
+// lanes 0-3, 12-15, 20-23, 24-27, the next 4-11, 16-19, 28-31, then the same of the upper 32).
+// With lane = (c, r) = (lane / 16, lane % 16) a cycle holds c0 with r / 4 in {0, 3} and c0 + 1
+// with r / 4 in {1, 2}, or the other way round, r % 4 taking all its values.  The tiles have no
+// padding; a lane reads 16-byte piece (logical piece) ^ swizzle of its row instead, and the
+// swizzle is such that a cycle's sixteen lanes hit the sixteen 16-byte columns of the banks:
+//   Q4(q) for q = r / 4: 0, 2, 3, 1, so that c ^ Q4 differs between the four (c, r / 4) of a cycle;
+//   V^T rows are 64 bytes (32 keys): element e uses Q4((e / 4) % 4); e % 4 picks the columns 4 (e % 4) ..
+//   K rows are 64 DK bytes, key j = 8 (r / 4) + 4 x + r % 4 of the step: the low bits of j
+//   choose among what the row's own offset leaves the same: none for odd DK (rows 64 bytes
+//   apart mod 256), bit 1 for DK = 2, 6 (128 bytes), bits 1 and 0 for DK = 4, 8 (0 bytes).
+#define Q4(q) ((((q) >> 1) & 1) | ((((q) ^ ((q) >> 1)) & 1) << 1))
+#define K_SWIZZLE(j, DK) ((Q4(((j) >> 3) & 3) | ((((j) >> 1) & 1) << 2) | (((j) & 1) << 3)) & ((DK) % 4 == 0 ? 15 : (DK) % 2 == 0 ? 7 : 3))
+#define V_SWIZZLE(e) Q4(((e) >> 2) & 3)
 
 // What one lane knows about the query row it serves (row = lane % 16 of a 16-row tile).
 struct RowInfo {
@@ -845,10 +860,10 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 // and V^T are copied from the pages into LDS once per workgroup (all threads; two tiles are on
 // their way while one is multiplied) and every wavefront reads its matrix-core operands from
 // there: the rows of a workgroup share one pass over the keys.
-//   LDS K tile:   [32 keys][D + 8]   (the 16-byte pad spreads a column of keys over the banks)
-//   LDS V^T tile: [D][32 keys + 8]
+//   LDS K tile:   [32 keys][D]    LDS V^T tile: [D][32 keys]
+// both without padding, the 16-byte pieces of a row XOR-swizzled (K_SWIZZLE, V_SWIZZLE).
 // Heads of 128 elements skip the registers: global_load_lds_dwordx4 writes the tiles into LDS
-// directly (three unpadded, XOR-swizzled buffers; see the DMA branch of the kernel).
+// directly (three buffers; see the DMA branch of the kernel).
 // row tiles per wavefront: two while the accumulators fit the register file
 #ifndef PRE_WAVES
 #define PRE_WAVES 4
@@ -871,12 +886,9 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     constexpr int D = DK * 32;
     static_assert(PRE_RT <= PRE_RT_OF(DK), "the accumulators of two row tiles fit the registers up to heads of 128");
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
-    constexpr int KROW = D + 8;       // elements per key row in LDS
-    constexpr int VROW = KSTEP + 8;   // elements per value-element row in LDS: 16-byte pieces stay aligned
-    constexpr int TILE = KSTEP * KROW + D * VROW;
     constexpr bool DMA = DK == 4 && PRE_WAVES == 4;  // tiles straight into LDS (measured 4-5 % faster)
-    constexpr int DTILE = 2 * KSTEP * D;  // elements of a tile without padding: K [32][D], then V^T [D][32]
-    __shared__ __attribute__((aligned(16))) bf16_t lds[DMA ? 3 * DTILE : 2 * TILE];
+    constexpr int TILE = 2 * KSTEP * D;  // elements of a tile: K [32 keys][D], then V^T [D][32 keys]
+    __shared__ __attribute__((aligned(16))) bf16_t lds[(DMA ? 3 : 2) * TILE];
 
     // the kv head varies fastest: workgroups go to the eight dies in turn, each die has an L2 of
     // its own, and this way a die sees the K/V of few heads, which the row blocks of a head share
@@ -927,6 +939,10 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     }
     RowState<DK, PRE_RT> st;
     init_rows<DK, PRE_RT>(st, row);
+    // what this lane reads from a tile in LDS: its two keys of a step and their swizzles
+    const int kx[2] = {KEY_OF_ROW(r16, 0), KEY_OF_ROW(r16, 1)};
+    const int ksw[2] = {K_SWIZZLE(kx[0], DK), K_SWIZZLE(kx[1], DK)};
+    const int vsw = V_SWIZZLE(r16);
 
     const int64_t k_head = (int64_t)kvh * P * D;
     const int64_t v_head = ((int64_t)nkv + kvh) * P * D;
@@ -972,8 +988,9 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         const int half = (threadIdx.x + PRE_WAVES * LLE_WAVE * i) / (2 * D);
         k_thread[i] = (q / (D / 8)) * D + (q % (D / 8)) * 8;
         v_thread[i] = (q / 2) * P + (q % 2) * 8;
-        k_lds[i] = (16 * half + q / (D / 8)) * KROW + (q % (D / 8)) * 8;
-        v_lds[i] = KSTEP * KROW + (q / 2) * VROW + 16 * half + (q % 2) * 8;
+        const int key = 16 * half + q / (D / 8);
+        k_lds[i] = key * D + (((q % (D / 8)) ^ K_SWIZZLE(key, DK)) * 8);
+        v_lds[i] = KSTEP * D + (q / 2) * KSTEP + (((2 * half + q % 2) ^ V_SWIZZLE(q / 2)) * 8);
     }
     auto fetch = [&](auto set_c) {
         constexpr int set = decltype(set_c)::value;
@@ -1013,11 +1030,12 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         fetch(std::integral_constant<int, 1 - set>{});  // tile step + 2
         if (step >= my_first && step < my_end) {
             const bf16_t* kt = lds + buf * TILE;
-            const bf16_t* vt = kt + KSTEP * KROW;
+            const bf16_t* vt = kt + KSTEP * D;
             tile_step<DK, PRE_RT>(
                 st, row,
-                [&](int x, int ks) { return *(const bf16x8*)(kt + KEY_OF_ROW(r16, x) * KROW + 32 * ks + 8 * c); },
-                [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * VROW + 8 * c); }, step * KSTEP, scale_log2);
+                [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ ksw[x]) * 8)); },
+                [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * KSTEP + ((c ^ vsw) * 8)); },
+                step * KSTEP, scale_log2);
         }
         stash(buf ^ 1, set_c);
         __syncthreads();
@@ -1025,14 +1043,12 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
 
     if constexpr (DMA) {
         // Tiles go from the pages straight into LDS (no registers, no stores by the wavefronts):
-        // a wavefront's load writes 1 KB of LDS in lane order (M0 holds where), so the tiles have
-        // no padding, and the 16-byte pieces of a row are XOR-swizzled instead, by which piece
-        // each lane fetches.  The loads are written in assembly so that the waits are ours: the
+        // a wavefront's load writes 1 KB of LDS in lane order (M0 holds where), so the swizzle is
+        // in which piece each lane fetches: the logical piece that belongs at its place (physical
+        // piece ^ swizzle).  The loads are written in assembly so that the waits are ours: the
         // compiler, seeing such a load, waits for ALL outstanding loads before every barrier.
         // vmcnt counts them in issue order, so "at most the 4 newest outstanding" means that
         // every tile requested before the last one has landed, whatever else was issued.
-        //   K  [32 keys][16 pieces]: logical piece p of key j at piece p ^ (j % 16)
-        //   V^T [D][4 pieces]:       logical piece p (keys 8p..8p+7) of element e at piece p ^ ((e / 4) % 4)
         // Three buffers: tile N is multiplied, N + 1 has landed or lands, N + 2 is requested.
         const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)lds;
         const int tid = threadIdx.x;
@@ -1041,10 +1057,10 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int q = tid + 256 * i;
-            const int key = q / 16, pk = q % 16;  // K: this half's key (i = half), physical piece
-            kd_thread[i] = (int64_t)(key % 16) * D + ((pk ^ (key % 16)) * 8);
+            const int key = q / 16, pk = q % 16;  // K: key of the step (half i), physical piece
+            kd_thread[i] = (int64_t)(key % 16) * D + ((pk ^ K_SWIZZLE(key, DK)) * 8);
             const int e = q / 4, pv = q % 4;
-            const int lp = pv ^ ((e / 4) % 4);  // logical piece: keys 8 lp .. 8 lp + 7 of the step
+            const int lp = pv ^ V_SWIZZLE(e);  // logical piece: keys 8 lp .. 8 lp + 7 of the step
             vd_half[i] = lp / 2;
             vd_thread[i] = (int64_t)e * P + (lp % 2) * 8;
         }
@@ -1055,23 +1071,21 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
             for (int i = 0; i < 2; ++i) {
                 const bf16_t* kp = (i ? half1 : half0) + k_head + (int64_t)(i ? page_off[1] : page_off[0]) * D + kd_thread[i];
                 const bf16_t* vp = (vd_half[i] ? half1 : half0) + v_head + (vd_half[i] ? page_off[1] : page_off[0]) + vd_thread[i];
-                const unsigned kdst = __builtin_amdgcn_readfirstlane(lds_base + 2 * (buf * DTILE + (wave * 64 + 256 * i) * 8));
+                const unsigned kdst = __builtin_amdgcn_readfirstlane(lds_base + 2 * (buf * TILE + (wave * 64 + 256 * i) * 8));
                 const unsigned vdst = kdst + 2 * KSTEP * D;
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(kdst), "v"(kp) : "memory", "m0");
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(vdst), "v"(vp) : "memory", "m0");
             }
             lookup();
         };
-        const int kx[2] = {KEY_OF_ROW(r16, 0), KEY_OF_ROW(r16, 1)};
-        const int vsw = (r16 / 4) % 4;
         auto dma_step = [&](int step, int buf, int next_buf) {
             dma(next_buf);  // tile step + 2
             if (step >= my_first && step < my_end) {
-                const bf16_t* kt = lds + buf * DTILE;
+                const bf16_t* kt = lds + buf * TILE;
                 const bf16_t* vt = kt + KSTEP * D;
                 tile_step<DK, PRE_RT>(
                     st, row,
-                    [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ (kx[x] % 16)) * 8)); },
+                    [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ ksw[x]) * 8)); },
                     [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * KSTEP + ((c ^ vsw) * 8)); },
                     step * KSTEP, scale_log2);
             }
