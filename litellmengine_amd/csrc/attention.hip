@@ -267,8 +267,9 @@ __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&
             lo_max = max(lo_max, __shfl_xor(lo_max, off, LLE_WAVE));
             pos_min = min(pos_min, __shfl_xor(pos_min, off, LLE_WAVE));
         }
-        st.open_lo[t] = lo_max;
-        st.open_hi[t] = pos_min == 0x7fffffff ? -1 : pos_min;
+        // (the same in every lane: kept in scalar registers, so that the test is a scalar branch)
+        st.open_lo[t] = __builtin_amdgcn_readfirstlane(lo_max);
+        st.open_hi[t] = __builtin_amdgcn_readfirstlane(pos_min == 0x7fffffff ? -1 : pos_min);
     }
     // The rows of Q are waited for here, once.  Left pending, their first use lies inside the
     // key loop, where the wait for them also waits for the K/V loads just issued for a later
@@ -279,6 +280,20 @@ __device__ __forceinline__ void init_rows(RowState<DK, RT>& st, const RowInfo (&
 #pragma unroll
             for (int ks = 0; ks < DK; ++ks) asm volatile("" : "+v"(st.qv[t][ks]));
     }
+}
+
+// The largest of eight scores, none of which is a NaN (masked scores are NEG_BIG, not infinite).
+// Written with the instruction itself: from fmaxf the compiler first passes every operand that a
+// select may have produced through an instruction of its own (x = max(x, x), which quiets a
+// signalling NaN), 8 + 7 instructions for what takes 4.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max_of_8(const float (&x)[8]) {
+    const float a = max3(x[0], x[1], x[2]), b = max3(x[3], x[4], x[5]);
+    return max3(max3(x[6], x[7], a), b, b);
 }
 
 // One 32-key step for RT tiles of 16 rows.  load_k(x, ks): for lane (c, r16) key
@@ -325,9 +340,7 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
                 if (j < row[t].lo || j > row[t].pos) x[t][i] = NEG_BIG;
             }
         }
-        const float top = fmaxf(fmaxf(fmaxf(x[t][0], x[t][1]), fmaxf(x[t][2], x[t][3])),
-                                fmaxf(fmaxf(x[t][4], x[t][5]), fmaxf(x[t][6], x[t][7])));
-        raise = raise || top > LAZY_MAX;
+        raise = raise || max_of_8(x[t]) > LAZY_MAX;
     }
     if (__builtin_amdgcn_ballot_w64(raise) != 0) {
 #pragma unroll
@@ -336,8 +349,7 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
             float sc[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) sc[i] = x[t][i] <= NEG_BIG ? NEG_BIG : s[t][i / 4][i % 4] * scale_log2;
-            float tile_max = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                                   fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+            float tile_max = max_of_8(sc);
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, LLE_WAVE));
             tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, LLE_WAVE));
             const float new_m = fmaxf(st.m[t], tile_max);
@@ -356,14 +368,15 @@ __device__ __forceinline__ void tile_step(RowState<DK, RT>& st, const RowInfo (&
     bf16x8 pb[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
-        float psum = 0.f;
+        // two chains of additions instead of one: a dependent addition waits for the one before it
+        float psum[2] = {0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float p = __builtin_amdgcn_exp2f(x[t][i]);
-            psum += p;
+            psum[i % 2] += p;
             pb[t][i] = (bf16_t)p;
         }
-        st.l[t] += psum;
+        st.l[t] += psum[0] + psum[1];
     }
 #pragma unroll
     for (int n = 0; n < 2 * DK; ++n) {
@@ -1052,32 +1065,36 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         // Three buffers: tile N is multiplied, N + 1 has landed or lands, N + 2 is requested.
         const unsigned lds_base = (unsigned)(size_t)(__attribute__((address_space(3))) void*)lds;
         const int tid = threadIdx.x;
-        int64_t kd_thread[2], vd_thread[2];
-        int vd_half[2];
+        // A load's address is a base that is the same for the whole wavefront (scalar registers:
+        // the page of one 16-key half) plus a byte offset per lane that never changes:
+        //   K:   half i of the step, key q / 16 of it, physical piece q % 16        (q = thread + 256 i)
+        //   V^T: half i of the step, element thread / 2, keys 8 (thread % 2) .. + 7 of the half
+        // so V^T lies in LDS as [half][D][16 keys]: rows of 32 bytes, which the sixteen lanes that
+        // a 16-byte read serves in a cycle (c0 and c0 + 1 of one half, eight different elements
+        // mod 8 each) spread over the sixteen columns of the banks without a swizzle.
+        unsigned kd_lane[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int q = tid + 256 * i;
-            const int key = q / 16, pk = q % 16;  // K: key of the step (half i), physical piece
-            kd_thread[i] = (int64_t)(key % 16) * D + ((pk ^ K_SWIZZLE(key, DK)) * 8);
-            const int e = q / 4, pv = q % 4;
-            const int lp = pv ^ V_SWIZZLE(e);  // logical piece: keys 8 lp .. 8 lp + 7 of the step
-            vd_half[i] = lp / 2;
-            vd_thread[i] = (int64_t)e * P + (lp % 2) * 8;
+            const int key = q / 16, pk = q % 16;
+            kd_lane[i] = 2u * (unsigned)((key % 16) * D + ((pk ^ K_SWIZZLE(key, DK)) * 8));
         }
+        const unsigned vd_lane = 2u * (unsigned)((tid / 2) * P + (tid % 2) * 8);
         auto dma = [&](int buf) {
-            const bf16_t* half0 = kv_layer + (int64_t)page_id[0] * page_stride;
-            const bf16_t* half1 = kv_layer + (int64_t)page_id[1] * page_stride;
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                const bf16_t* kp = (i ? half1 : half0) + k_head + (int64_t)(i ? page_off[1] : page_off[0]) * D + kd_thread[i];
-                const bf16_t* vp = (vd_half[i] ? half1 : half0) + v_head + (vd_half[i] ? page_off[1] : page_off[0]) + vd_thread[i];
+                // (a page's offset as an unsigned 32 x 32 -> 64 bit product: two scalar instructions)
+                const bf16_t* page = kv_layer + (uint64_t)(uint32_t)page_id[i] * (uint64_t)(uint32_t)page_stride;
+                const bf16_t* kb = page + k_head + (int64_t)page_off[i] * D;
+                const bf16_t* vb = page + v_head + page_off[i];
                 const unsigned kdst = __builtin_amdgcn_readfirstlane(lds_base + 2 * (buf * TILE + (wave * 64 + 256 * i) * 8));
                 const unsigned vdst = kdst + 2 * KSTEP * D;
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(kdst), "v"(kp) : "memory", "m0");
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(vdst), "v"(vp) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(kdst), "v"(kd_lane[i]), "s"(kb) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(vdst), "v"(vd_lane), "s"(vb) : "memory", "m0");
             }
             lookup();
         };
+        const int v_read = (c / 2) * (D * 16) + r16 * 16 + (c % 2) * 8;  // this lane's place in V^T for n = 0
         auto dma_step = [&](int step, int buf, int next_buf) {
             dma(next_buf);  // tile step + 2
             if (step >= my_first && step < my_end) {
@@ -1086,8 +1103,7 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
                 tile_step<DK, PRE_RT>(
                     st, row,
                     [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ ksw[x]) * 8)); },
-                    [&](int n) { return *(const bf16x8*)(vt + (16 * n + r16) * KSTEP + ((c ^ vsw) * 8)); },
-                    step * KSTEP, scale_log2);
+                    [&](int n) { return *(const bf16x8*)(vt + v_read + n * 256); }, step * KSTEP, scale_log2);
             }
             // the four loads just issued may stay in flight; the tile before them has landed
             asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
@@ -1542,7 +1558,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 int prefill_row_tiles, const FusedQKV& fused, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
-    if (S > 65535 || nkv > 65535) return (int)hipErrorInvalidValue;
+    if (S > 65535 || nkv > 65535 || page_stride < 0 || page_stride >= ((int64_t)1 << 32)) return (int)hipErrorInvalidValue;
     if (nsplit_decode < 1 || nsplit_decode > 64 || nsplit_prefill < 1 || nsplit_prefill > 64)
         return (int)hipErrorInvalidValue;
     const float scale_log2 = scale * 1.44269504088896340736f;
