@@ -866,29 +866,32 @@ __global__ __launch_bounds__(LLE_WAVE) void mfma_combine_kernel(const float* __r
 }
 
 // Requests with more than 16 rows.  grid = (kv heads, row blocks x key splits, requests); a
-// workgroup takes 128 rows (64 for heads over 128 elements), each of its four wavefronts 32
-// (16) of them; two workgroups fit a CU (256 registers a lane each), which measured faster
-// than one of twice the size: a heavy and a light row block then share a CU.  A short portion after a long past has few row blocks: its keys are then split
-// over `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K
-// and V^T are copied from the pages into LDS once per workgroup (all threads; two tiles are on
-// their way while one is multiplied) and every wavefront reads its matrix-core operands from
-// there: the rows of a workgroup share one pass over the keys.
+// workgroup takes a block of rows (token, head of the group) and walks the keys they see in steps
+// of 32.  A short portion after a long past has few row blocks: its keys are then split over
+// `nsplit` workgroups, which leave (m, l, acc) for the combine kernel.  The 32-key tiles of K and
+// V^T are copied from the pages into LDS once per workgroup (all threads; two tiles are on their
+// way while one is multiplied) and every wavefront reads its matrix-core operands from there:
+// the rows of a workgroup share one pass over the keys.
 //   LDS K tile:   [32 keys][D]    LDS V^T tile: [D][32 keys]
 // both without padding, the 16-byte pieces of a row XOR-swizzled (K_SWIZZLE, V_SWIZZLE).
 // Heads of 128 elements skip the registers: global_load_lds_dwordx4 writes the tiles into LDS
 // directly (three buffers; see the DMA branch of the kernel).
-// row tiles per wavefront: two while the accumulators fit the register file
-#ifndef PRE_WAVES
-#define PRE_WAVES 4
-#endif
+// The shapes of a workgroup (PRE_WAVES wavefronts of PRE_RT tiles of 16 rows each):
+//   4 x 1: 64 rows.  Twice the workgroups of half the height: for launches so small that these
+//          all fit the chip at once.
+//   4 x 2: 128 rows; every operand read from LDS serves both tiles of a wavefront.  Two
+//          workgroups a CU in 256 registers a lane (heads up to 128; above, 4 x 1 only).
+//   8 x 1: 128 rows, heads of 128 only.  Two workgroups a CU are four wavefronts a SIMD, in 128
+//          registers each.  A wavefront issues about one instruction in eight cycles whatever
+//          its kind, and a matrix instruction holds it for sixteen; the wavefronts of a SIMD run
+//          side by side until they meet at an issue port, so four of them get more out of it
+//          than two (measured: 118 against 128 us for 2048 rows over 4096 keys), although each
+//          tile is then read from LDS by twice as many wavefronts.
 #ifndef PRE_RT_MAX
 #define PRE_RT_MAX 2
 #endif
 #define PRE_RT_OF(DK) ((DK) <= 4 ? PRE_RT_MAX : 1)
-// PRE_RT row tiles per wavefront: two share every operand that is read from LDS; one gives twice the
-// workgroups of half the height, which fills the chip better when a launch is only one round of
-// them and the causal mask makes them unequal (a prompt from its first token).
-template <int DK, int PRE_RT>
+template <int DK, int PRE_RT, int PRE_WAVES = 4>
 // (heads over 192 elements need more than the 256 registers a lane that two workgroups a CU leave)
 __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ kv_layer, const int32_t* __restrict__ block_tables,
@@ -899,7 +902,8 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     constexpr int D = DK * 32;
     static_assert(PRE_RT <= PRE_RT_OF(DK), "the accumulators of two row tiles fit the registers up to heads of 128");
     constexpr int PRE_ROWS = PRE_WAVES * 16 * PRE_RT;
-    constexpr bool DMA = DK == 4 && PRE_WAVES == 4;  // tiles straight into LDS (measured 4-5 % faster)
+    constexpr bool DMA = DK == 4 && (PRE_WAVES == 4 || PRE_WAVES == 8);  // tiles straight into LDS (measured 4-5 % faster)
+    static_assert(PRE_WAVES == 4 || (DK == 4 && PRE_RT == 1), "eight wavefronts: heads of 128, one row tile each");
     constexpr int TILE = 2 * KSTEP * D;  // elements of a tile: K [32 keys][D], then V^T [D][32 keys]
     __shared__ __attribute__((aligned(16))) bf16_t lds[(DMA ? 3 : 2) * TILE];
 
@@ -950,6 +954,9 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         my_first = my_lo / KSTEP;
         my_end = min(end_step, (past + my_last_row / G) / KSTEP + 1);
     }
+    // (the same in every lane of a wavefront: in scalar registers the tests on them are scalar branches)
+    my_first = __builtin_amdgcn_readfirstlane(my_first);
+    my_end = __builtin_amdgcn_readfirstlane(my_end);
     RowState<DK, PRE_RT> st;
     init_rows<DK, PRE_RT>(st, row);
     // what this lane reads from a tile in LDS: its two keys of a step and their swizzles
@@ -973,7 +980,8 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
     // is no constant).  A half wholly outside [lo_min, hi] may lie in a page that is not there:
     // the page index is clamped to those of keys that are.
     const int page_lo = lo_min / P, page_hi = hi / P;
-    int look_page = (first_step * KSTEP) / P, look_off = (first_step * KSTEP) % P;
+    int look_page = __builtin_amdgcn_readfirstlane((first_step * KSTEP) / P);
+    int look_off = __builtin_amdgcn_readfirstlane((first_step * KSTEP) % P);
     int page_id[2], page_off[2];
     auto lookup = [&]() {
 #pragma unroll
@@ -1072,46 +1080,63 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
         // so V^T lies in LDS as [half][D][16 keys]: rows of 32 bytes, which the sixteen lanes that
         // a 16-byte read serves in a cycle (c0 and c0 + 1 of one half, eight different elements
         // mod 8 each) spread over the sixteen columns of the banks without a swizzle.
-        unsigned kd_lane[2];
+        constexpr int LOADS = 512 / (PRE_WAVES * LLE_WAVE);  // of K and of V^T, per thread and tile
+        unsigned kd_lane[LOADS], vd_lane[LOADS];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int q = tid + 256 * i;
+        for (int i = 0; i < LOADS; ++i) {
+            const int q = tid + PRE_WAVES * LLE_WAVE * i;  // the half is q / 256: the same for a wavefront's load
             const int key = q / 16, pk = q % 16;
             kd_lane[i] = 2u * (unsigned)((key % 16) * D + ((pk ^ K_SWIZZLE(key, DK)) * 8));
+            vd_lane[i] = 2u * (unsigned)(((q % 256) / 2) * P + (q % 2) * 8);
         }
-        const unsigned vd_lane = 2u * (unsigned)((tid / 2) * P + (tid % 2) * 8);
         auto dma = [&](int buf) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < LOADS; ++i) {
+                const int first_piece = __builtin_amdgcn_readfirstlane(wave * LLE_WAVE + PRE_WAVES * LLE_WAVE * i);
+                const int half = first_piece / 256;
                 // (a page's offset as an unsigned 32 x 32 -> 64 bit product: two scalar instructions)
-                const bf16_t* page = kv_layer + (uint64_t)(uint32_t)page_id[i] * (uint64_t)(uint32_t)page_stride;
-                const bf16_t* kb = page + k_head + (int64_t)page_off[i] * D;
-                const bf16_t* vb = page + v_head + page_off[i];
-                const unsigned kdst = __builtin_amdgcn_readfirstlane(lds_base + 2 * (buf * TILE + (wave * 64 + 256 * i) * 8));
+                const bf16_t* page = kv_layer + (uint64_t)(uint32_t)(half ? page_id[1] : page_id[0]) * (uint64_t)(uint32_t)page_stride;
+                const int off = half ? page_off[1] : page_off[0];
+                const bf16_t* kb = page + k_head + (int64_t)off * D;
+                const bf16_t* vb = page + v_head + off;
+                const unsigned kdst = lds_base + 2 * (buf * TILE + first_piece * 8);
                 const unsigned vdst = kdst + 2 * KSTEP * D;
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(kdst), "v"(kd_lane[i]), "s"(kb) : "memory", "m0");
-                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(vdst), "v"(vd_lane), "s"(vb) : "memory", "m0");
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(vdst), "v"(vd_lane[i]), "s"(vb) : "memory", "m0");
             }
             lookup();
         };
         const int v_read = (c / 2) * (D * 16) + r16 * 16 + (c % 2) * 8;  // this lane's place in V^T for n = 0
         auto dma_step = [&](int step, int buf, int next_buf) {
+            // the key operands are asked for first: the scalar arithmetic of the loads' addresses
+            // then covers their way from LDS
+            const bf16_t* kt = lds + buf * TILE;
+            const bf16_t* vt = kt + KSTEP * D;
+            bf16x8 kreg[2][DK];
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int ks = 0; ks < DK; ++ks)
+                    kreg[x][ks] = *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ ksw[x]) * 8));
             dma(next_buf);  // tile step + 2
             if (step >= my_first && step < my_end) {
-                const bf16_t* kt = lds + buf * TILE;
-                const bf16_t* vt = kt + KSTEP * D;
                 tile_step<DK, PRE_RT>(
-                    st, row,
-                    [&](int x, int ks) { return *(const bf16x8*)(kt + kx[x] * D + (((4 * ks + c) ^ ksw[x]) * 8)); },
+                    st, row, [&](int x, int ks) { return kreg[x][ks]; },
                     [&](int n) { return *(const bf16x8*)(vt + v_read + n * 256); }, step * KSTEP, scale_log2);
             }
-            // the four loads just issued may stay in flight; the tile before them has landed
-            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            // the loads just issued may stay in flight; the tile before them has landed
+            if constexpr (LOADS == 2)
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
             __builtin_amdgcn_s_barrier();
         };
         dma(0);  // tile first_step
         dma(1);  // tile first_step + 1
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        if constexpr (LOADS == 2)
+            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         for (int step = first_step; step < end_step; step += 3) {
             dma_step(step, 0, 2);
@@ -1486,7 +1511,7 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
                        const int32_t* token_seq, bf16_t* out, float* ws_o, float* ws_ml, int N, int S, int nq,
                        int nkv, int P, int64_t page_stride, int max_pages, int window, float scale_log2,
                        int run_decode, int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                       int prefill_row_tiles, const FusedQKV& fused, hipStream_t stream) {
+                       int prefill_form, const FusedQKV& fused, hipStream_t stream) {
     constexpr int D = DK * 32;
     const int G = nq / nkv;
     if (!run_decode) nsplit_decode = 1;
@@ -1523,19 +1548,23 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
     }
     if (run_prefill) {
         const int rows = max_q_len * G;
-        auto launch = [&](auto rt) {
-            constexpr int RT = decltype(rt)::value;
-            constexpr int PRE_ROWS = PRE_WAVES * 16 * RT;
+        auto launch = [&](auto rt, auto waves) {
+            constexpr int RT = decltype(rt)::value, WAVES = decltype(waves)::value;
+            constexpr int PRE_ROWS = WAVES * 16 * RT;
             const int blocks = (rows + PRE_ROWS - 1) / PRE_ROWS;
             const int64_t workgroups = (int64_t)nkv * blocks * nsplit_prefill * S;
-            mfma_prefill_kernel<DK, RT><<<dim3(nkv, blocks * nsplit_prefill, S), PRE_WAVES * LLE_WAVE, 0, stream>>>(
+            mfma_prefill_kernel<DK, RT, WAVES><<<dim3(nkv, blocks * nsplit_prefill, S), WAVES * LLE_WAVE, 0, stream>>>(
                 q, kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, out, ws_o, ws_ml, ws_stride, nsplit_prefill,
                 nq, nkv, P, page_stride, max_pages, window, scale_log2, workgroups <= 2 * compute_units() ? 1 : 0);
         };
-        if (PRE_RT_OF(DK) == 1 || prefill_row_tiles == 1)
-            launch(std::integral_constant<int, 1>{});
-        else
-            launch(std::integral_constant<int, PRE_RT_OF(DK)>{});
+        using Four = std::integral_constant<int, 4>;
+        if (DK == 4 && prefill_form == 3) {
+            if constexpr (DK == 4) launch(std::integral_constant<int, 1>{}, std::integral_constant<int, 8>{});
+        } else if (PRE_RT_OF(DK) == 1 || prefill_form == 1) {
+            launch(std::integral_constant<int, 1>{}, Four{});
+        } else {
+            launch(std::integral_constant<int, PRE_RT_OF(DK)>{}, Four{});
+        }
     }
     if (lane && hipStreamWaitEvent(stream, lane->join, 0) != hipSuccess) return (int)hipGetLastError();
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
@@ -1555,7 +1584,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 void* ws_o, void* ws_ml, int N, int S, int nq, int nkv, int d, int page_size,
                                 int64_t page_stride, int max_pages, int window, float scale, int run_decode,
                                 int nsplit_decode, int run_prefill, int nsplit_prefill, int max_q_len,
-                                int prefill_row_tiles, const FusedQKV& fused, hipStream_t stream) {
+                                int prefill_form, const FusedQKV& fused, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d % 32 != 0 || d > 256 || page_size % 16 != 0 || nq % nkv != 0) return (int)hipErrorInvalidValue;
     if (S > 65535 || nkv > 65535 || page_stride < 0 || page_stride >= ((int64_t)1 << 32)) return (int)hipErrorInvalidValue;
@@ -1568,7 +1597,7 @@ static int paged_attention_mfma(const void* q, void* kv_layer, const void* block
                                 (const int32_t*)seq_slots, (const int32_t*)cu_tokens, (const int32_t*)kv_lens,      \
                                 (const int32_t*)token_seq, (bf16_t*)out, (float*)ws_o, (float*)ws_ml, N, S, nq, nkv, \
                                 page_size, page_stride, max_pages, window, scale_log2, run_decode, nsplit_decode,   \
-                                run_prefill, nsplit_prefill, max_q_len, prefill_row_tiles, fused, stream);
+                                run_prefill, nsplit_prefill, max_q_len, prefill_form, fused, stream);
     switch (d / 32) {
         LLE_ATT_CASE(1)
         LLE_ATT_CASE(2)
@@ -1588,12 +1617,12 @@ extern "C" int lle_paged_attention_mfma(const void* q, const void* kv_layer, con
                                         const void* token_seq, void* out, void* ws_o, void* ws_ml, int N, int S,
                                         int nq, int nkv, int d, int page_size, int64_t page_stride, int max_pages,
                                         int window, float scale, int run_decode, int nsplit_decode, int run_prefill,
-                                        int nsplit_prefill, int max_q_len, int prefill_row_tiles,
+                                        int nsplit_prefill, int max_q_len, int prefill_form,
                                         hipStream_t stream) {
     const FusedQKV none = {};
     return paged_attention_mfma(q, (void*)kv_layer, block_tables, seq_slots, cu_tokens, kv_lens, token_seq, out, ws_o,
                                 ws_ml, N, S, nq, nkv, d, page_size, page_stride, max_pages, window, scale, run_decode,
-                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, prefill_row_tiles, none, stream);
+                                nsplit_decode, run_prefill, nsplit_prefill, max_q_len, prefill_form, none, stream);
 }
 
 // Decode steps only (every request has at most 16 / group tokens), head_dim a multiple of 64, a

@@ -327,7 +327,7 @@ class HipOps:
         run_prefill = max_q_len * group > 16
         ns_decode = self.decode_splits(S, nkv, max_kv_len, win) if run_decode else 1
         ns_prefill = self.prefill_splits(S, nkv, group, d, max_q_len, max_kv_len, win) if run_prefill else 1
-        row_tiles = (self.prefill_row_tiles(S, nkv, group, d, max_q_len, max_kv_len, win, ns_prefill, q.device)
+        row_tiles = (self.prefill_form(S, nkv, group, d, max_q_len, max_kv_len, win, ns_prefill, q.device)
                      if run_prefill else 0)
         ns = max(ns_decode, ns_prefill)
         ws_o = ws_ml = None
@@ -398,7 +398,7 @@ class HipOps:
         return out
 
     force_generic_attention = False  # tests flip this to compare the two families of kernels
-    force_prefill_row_tiles = 0      # tests set 1 or 2 to reach both heights of the prompt-portion workgroups
+    force_prefill_form = 0           # tests set 1, 2 or 3 to reach every shape of the prompt-portion workgroups
     force_separate_rope = False      # tests flip this to compare the fused decode step with its two halves
     # measured on MI355X: about one workgroup per CU and at least 8 32-key steps (two per
     # wavefront) per split are best; more splits cost more in partial results than they gain
@@ -421,29 +421,30 @@ class HipOps:
 
     _compute_units: dict = {}
 
-    def prefill_row_tiles(self, num_seqs: int, num_kv_heads: int, group: int, head_dim: int, max_q_len: int,
-                          max_kv_len: int, window: int, nsplit: int, device) -> int:
-        """Tiles of 16 rows per wavefront of the prompt-portion kernel: 2 (128 rows a workgroup; every
-        operand read from LDS serves both) unless the launch is so small that workgroups of 64 rows
-        still fit the chip at once, or is one round of unequal workgroups (a prompt from its first
-        tokens under the causal mask, no window): then 1.  Measured on MI355X at heads of 128: a
-        2048-token prompt 58 against 65 us, 1500 tokens 42 against 54; with a past of half the
-        portion or more the taller workgroups win by 20-30 %."""
+    def prefill_form(self, num_seqs: int, num_kv_heads: int, group: int, head_dim: int, max_q_len: int,
+                     max_kv_len: int, window: int, nsplit: int, device) -> int:
+        """The shape of the prompt-portion kernel's workgroups:
+          1: four wavefronts of one 16-row tile each (64 rows a workgroup),
+          2: four wavefronts of two tiles each (128 rows; every operand read from LDS serves both tiles),
+          3: eight wavefronts of one tile each (128 rows; four wavefronts a SIMD; heads of 128 only).
+        The low form when its workgroups all fit the chip at once (a short portion); else the tall
+        ones, which share a pass over the keys between more rows: form 3 at heads of 128, form 2
+        below.  Measured on MI355X at heads of 128 (forms 1 / 2 / 3): 2048 tokens from an empty cache
+        60 / 65 / 57 us, 2048 tokens after 2048 keys 148 / 128 / 118 us, 49 tokens after 2048 keys
+        17 / 21 / 19 us."""
         if head_dim > 128:
             return 1
-        if self.force_prefill_row_tiles:
-            return self.force_prefill_row_tiles
+        if self.force_prefill_form:
+            return self.force_prefill_form if head_dim == 128 or self.force_prefill_form < 3 else 2
         key = device.index if device.index is not None else torch.cuda.current_device()
         if key not in self._compute_units:
             self._compute_units[key] = torch.cuda.get_device_properties(key).multi_processor_count
         resident = 2 * self._compute_units[key]
         rows = max_q_len * group
-        per_block = num_kv_heads * max(1, num_seqs) * max(1, nsplit)
-        tall, low = -(-rows // 128) * per_block, -(-rows // 64) * per_block
-        past = max_kv_len - max_q_len
-        if low <= resident or (tall <= resident and not window and 8 * past <= max_q_len):
+        low = -(-rows // 64) * num_kv_heads * max(1, num_seqs) * max(1, nsplit)
+        if low <= resident:
             return 1
-        return 2
+        return 3 if head_dim == 128 else 2
 
     def f32_attention_splits(self, num_seqs: int, num_kv_heads: int, row_blocks: int, max_q_len: int,
                              max_kv_len: int, window: int) -> int:

@@ -411,18 +411,18 @@ def test_float32_matrix_core_attention(nq, nkv, d, P, window, lens):
 ])
 def test_matrix_core_attention(nq, nkv, d, P, window, lens):
     """The bfloat16 matrix-core kernels against the plain form and the generic kernel; prompt
-    portions with workgroups of both heights (one and two row tiles per wavefront)."""
+    portions with every shape of workgroup (four wavefronts of one or of two row tiles, eight of one)."""
     need = max((p + l + P - 1) // P for p, l in lens)
     args, mq, mk = attention_case(torch.bfloat16, nq, nkv, d, P, window, lens, pages=sum((p + l + P - 1) // P for p, l in lens) + 3,
                                   max_pages=need + 1)
     o = ops()
     want = REF.paged_attention(*args)
-    for row_tiles in (1, 2):
-        o.force_prefill_row_tiles = row_tiles
+    for row_tiles in (1, 2, 3):
+        o.force_prefill_form = row_tiles
         try:
             got = o.paged_attention(*args, *mq, mk)
         finally:
-            o.force_prefill_row_tiles = 0
+            o.force_prefill_form = 0
         err = (got.double() - want.double()).abs().max().item()
         assert err < 2e-2, (row_tiles, err)
     o.force_generic_attention = True
