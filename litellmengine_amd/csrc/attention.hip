@@ -1089,14 +1089,26 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
             kd_lane[i] = 2u * (unsigned)((key % 16) * D + ((pk ^ K_SWIZZLE(key, DK)) * 8));
             vd_lane[i] = 2u * (unsigned)(((q % 256) / 2) * P + (q % 2) * 8);
         }
+        // With one load of K and one of V^T per wavefront and tile a wavefront needs the page of
+        // its own half only, and follows that alone: half the scalar arithmetic a step.
+        int own_page = 0, own_off = 0, own_id = 0;
+        const int own_adv_pages = KSTEP / P, own_adv_off = KSTEP % P;
+        auto own_lookup = [&]() { own_id = table[__builtin_amdgcn_readfirstlane(min(max(own_page, page_lo), page_hi))]; };
+        if constexpr (LOADS == 1) {
+            const int key0 = first_step * KSTEP + 16 * (wave / 4);
+            own_page = __builtin_amdgcn_readfirstlane(key0 / P);
+            own_off = __builtin_amdgcn_readfirstlane(key0 % P);
+            own_lookup();
+        }
         auto dma = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < LOADS; ++i) {
                 const int first_piece = __builtin_amdgcn_readfirstlane(wave * LLE_WAVE + PRE_WAVES * LLE_WAVE * i);
                 const int half = first_piece / 256;
                 // (a page's offset as an unsigned 32 x 32 -> 64 bit product: two scalar instructions)
-                const bf16_t* page = kv_layer + (uint64_t)(uint32_t)(half ? page_id[1] : page_id[0]) * (uint64_t)(uint32_t)page_stride;
-                const int off = half ? page_off[1] : page_off[0];
+                const int id = LOADS == 1 ? own_id : (half ? page_id[1] : page_id[0]);
+                const bf16_t* page = kv_layer + (uint64_t)(uint32_t)id * (uint64_t)(uint32_t)page_stride;
+                const int off = LOADS == 1 ? own_off : (half ? page_off[1] : page_off[0]);
                 const bf16_t* kb = page + k_head + (int64_t)off * D;
                 const bf16_t* vb = page + v_head + off;
                 const unsigned kdst = lds_base + 2 * (buf * TILE + first_piece * 8);
@@ -1104,7 +1116,17 @@ __global__ __launch_bounds__(PRE_WAVES* LLE_WAVE, DK <= 6 ? 2 : 1) void mfma_pre
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(kdst), "v"(kd_lane[i]), "s"(kb) : "memory", "m0");
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(vdst), "v"(vd_lane[i]), "s"(vb) : "memory", "m0");
             }
-            lookup();
+            if constexpr (LOADS == 1) {
+                own_page += own_adv_pages;
+                own_off += own_adv_off;
+                if (own_off >= P) {
+                    own_off -= P;
+                    ++own_page;
+                }
+                own_lookup();
+            } else {
+                lookup();
+            }
         };
         const int v_read = (c / 2) * (D * 16) + r16 * 16 + (c % 2) * 8;  // this lane's place in V^T for n = 0
         auto dma_step = [&](int step, int buf, int next_buf) {
