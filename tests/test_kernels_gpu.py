@@ -400,7 +400,7 @@ def test_float32_matrix_core_attention(nq, nkv, d, P, window, lens):
 
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 32, 16, None), (16, 2, 64, 32, None),
                                                (6, 1, 96, 16, 40), (8, 2, 256, 16, None), (32, 8, 128, 16, 700),
-                                               (3, 1, 160, 48, None)])
+                                               (3, 1, 160, 48, None), (8, 2, 128, 48, None), (4, 1, 128, 32, 100)])
 @pytest.mark.parametrize("lens", [
     [(0, 9), (17, 1), (30, 2), (5, 11)],          # portions beside decoded tokens
     [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
