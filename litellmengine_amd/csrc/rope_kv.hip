@@ -173,6 +173,64 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_vec_kernel(
     }
 }
 
+// The V heads of many tokens into the transposed pages.  A workgroup takes 16 consecutive
+// tokens of the batch and one kv head: the rows are read whole into LDS, and every thread
+// writes one value element of 8 tokens, as one 16-byte store when those tokens sit in
+// consecutive slots of one page starting at a multiple of 8 (prompt portions do), else one by one.
+#define VW_TOKENS 16
+__device__ __forceinline__ void v_write_transposed_block(const bf16_t* __restrict__ qkv,
+                                                         const int32_t* __restrict__ slots,
+                                                         bf16_t* __restrict__ kv_layer, int N, int nq, int nkv, int d,
+                                                         int page_size, int64_t page_stride, int t0, int kvh,
+                                                         bf16_t* tile /* [VW_TOKENS][d + 2] */, int* s_slot) {
+    const int width = (nq + 2 * nkv) * d;
+    const int row = d + 2;
+    for (int idx = threadIdx.x; idx < VW_TOKENS * (d / 8); idx += blockDim.x) {
+        const int t = idx / (d / 8), ch = idx % (d / 8);
+        if (t0 + t < N) {
+            const rbf16x8 v = *(const rbf16x8*)(qkv + (int64_t)(t0 + t) * width + (int64_t)(nq + nkv + kvh) * d + 8 * ch);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tile[t * row + 8 * ch + i] = v[i];
+        }
+    }
+    if (threadIdx.x < VW_TOKENS) s_slot[threadIdx.x] = t0 + threadIdx.x < N ? slots[t0 + threadIdx.x] : -1;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 2 * d; idx += blockDim.x) {
+        const int g = idx / d, e = idx - g * d;  // tokens 8 g .. 8 g + 7, value element e
+        const int first = s_slot[8 * g];
+        bool run = first >= 0 && first % 8 == 0 && first % page_size + 8 <= page_size;
+#pragma unroll
+        for (int i = 1; i < 8; ++i) run = run && s_slot[8 * g + i] == first + i;
+        if (run) {
+            const int64_t page = first / page_size;
+            const int off = first - (int)page * page_size;
+            rbf16x8 y;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = tile[(8 * g + i) * row + e];
+            *(rbf16x8*)(kv_layer + page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off) = y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int slot = s_slot[8 * g + i];
+                if (slot < 0) continue;
+                const int64_t page = slot / page_size;
+                const int off = slot - (int)page * page_size;
+                kv_layer[page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off] =
+                    tile[(8 * g + i) * row + e];
+            }
+        }
+    }
+}
+__global__ __launch_bounds__(256) void v_write_transposed_kernel(const bf16_t* __restrict__ qkv,
+                                                                  const int32_t* __restrict__ slots,
+                                                                  bf16_t* __restrict__ kv_layer, int N, int nq, int nkv,
+                                                                  int d, int page_size, int64_t page_stride) {
+    extern __shared__ bf16_t tile[];  // [VW_TOKENS][d + 2]
+    __shared__ int s_slot[VW_TOKENS];
+    v_write_transposed_block(qkv, slots, kv_layer, N, nq, nkv, d, page_size, page_stride, blockIdx.x * VW_TOKENS,
+                             blockIdx.y, tile, s_slot);
+}
+
 // The same for a rotation over the whole head (rot == d): a lane holds four elements of the
 // low half and their four partners of the high half, so the rotation needs no exchange between
 // lanes, and one (cos, sin) pair serves both partners.
@@ -191,7 +249,17 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_pair_kernel(
     const bf16_t* __restrict__ qkv, const int32_t* __restrict__ slots, const void* __restrict__ q_weight,
     const void* __restrict__ k_weight, int weight_dtype, const float* __restrict__ cos_sin, float eps,
     bf16_t* __restrict__ q_out, bf16_t* __restrict__ kv_layer, int nq, int nkv, int d, int page_size,
-    int64_t page_stride, int write_kv, int total_heads) {
+    int64_t page_stride, int write_kv, int total_heads, int head_blocks, int N) {
+    // write_kv == 2: the workgroups after the first `head_blocks` take the V heads of 16 tokens and
+    // one kv head each into the transposed pages (the same launch: the two kinds of work overlap)
+    if ((int)blockIdx.x >= head_blocks) {
+        extern __shared__ bf16_t tile[];  // [VW_TOKENS][d + 2]
+        __shared__ int s_slot[VW_TOKENS];
+        const int vb = blockIdx.x - head_blocks;
+        v_write_transposed_block(qkv, slots, kv_layer, N, nq, nkv, d, page_size, page_stride, (vb / nkv) * VW_TOKENS,
+                                 vb % nkv, tile, s_slot);
+        return;
+    }
     const int lph = d / 8;  // lanes per head
     const int lane = threadIdx.x % LLE_WAVE;
     const int heads_per_wave = LLE_WAVE / lph;
@@ -268,57 +336,6 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_pair_kernel(
     }
 }
 
-// The V heads of many tokens into the transposed pages.  A workgroup takes 16 consecutive
-// tokens of the batch and one kv head: the rows are read whole into LDS, and every thread
-// writes one value element of 8 tokens, as one 16-byte store when those tokens sit in
-// consecutive slots of one page starting at a multiple of 8 (prompt portions do), else one by one.
-#define VW_TOKENS 16
-__global__ __launch_bounds__(256) void v_write_transposed_kernel(const bf16_t* __restrict__ qkv,
-                                                                  const int32_t* __restrict__ slots,
-                                                                  bf16_t* __restrict__ kv_layer, int N, int nq, int nkv,
-                                                                  int d, int page_size, int64_t page_stride) {
-    extern __shared__ bf16_t tile[];  // [VW_TOKENS][d + 2]
-    __shared__ int s_slot[VW_TOKENS];
-    const int t0 = blockIdx.x * VW_TOKENS, kvh = blockIdx.y;
-    const int width = (nq + 2 * nkv) * d;
-    const int row = d + 2;
-    for (int idx = threadIdx.x; idx < VW_TOKENS * (d / 8); idx += blockDim.x) {
-        const int t = idx / (d / 8), ch = idx % (d / 8);
-        if (t0 + t < N) {
-            const rbf16x8 v = *(const rbf16x8*)(qkv + (int64_t)(t0 + t) * width + (int64_t)(nq + nkv + kvh) * d + 8 * ch);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) tile[t * row + 8 * ch + i] = v[i];
-        }
-    }
-    if (threadIdx.x < VW_TOKENS) s_slot[threadIdx.x] = t0 + threadIdx.x < N ? slots[t0 + threadIdx.x] : -1;
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < 2 * d; idx += blockDim.x) {
-        const int g = idx / d, e = idx - g * d;  // tokens 8 g .. 8 g + 7, value element e
-        const int first = s_slot[8 * g];
-        bool run = first >= 0 && first % 8 == 0 && first % page_size + 8 <= page_size;
-#pragma unroll
-        for (int i = 1; i < 8; ++i) run = run && s_slot[8 * g + i] == first + i;
-        if (run) {
-            const int64_t page = first / page_size;
-            const int off = first - (int)page * page_size;
-            rbf16x8 y;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) y[i] = tile[(8 * g + i) * row + e];
-            *(rbf16x8*)(kv_layer + page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off) = y;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int slot = s_slot[8 * g + i];
-                if (slot < 0) continue;
-                const int64_t page = slot / page_size;
-                const int off = slot - (int)page * page_size;
-                kv_layer[page * page_stride + ((int64_t)nkv + kvh) * page_size * d + (int64_t)e * page_size + off] =
-                    tile[(8 * g + i) * row + e];
-            }
-        }
-    }
-}
-
 // cos and sin of float(pos) * inv_freq[i] for every token of the step: out [N][half][2]
 __global__ __launch_bounds__(256) void rope_table_kernel(const int32_t* __restrict__ positions,
                                                           const float* __restrict__ inv_freq,
@@ -354,11 +371,20 @@ extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* slots,
         const int blocks = (total_heads + heads_per_block - 1) / heads_per_block;
         // many tokens: V goes through the transposing kernel (16-byte stores into the pages)
         const bool split_v = write_kv && N >= 64 && page_size % 8 == 0 && (N + VW_TOKENS - 1) / VW_TOKENS <= 0x7fffffff;
+        const int64_t v_blocks = split_v ? (int64_t)((N + VW_TOKENS - 1) / VW_TOKENS) * nkv : 0;
+        if (rot == d && blocks + v_blocks <= 0x7fffffff) {
+            qk_norm_rope_write_pair_kernel<<<(unsigned)(blocks + v_blocks), 256,
+                                             split_v ? VW_TOKENS * (d + 2) * sizeof(bf16_t) : 0, stream>>>(
+                (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, eps,
+                (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
+                write_kv ? (split_v ? 2 : 1) : 0, total_heads, blocks, N);
+            LLE_RETURN_LAUNCH_STATUS();
+        }
         if (rot == d)
             qk_norm_rope_write_pair_kernel<<<blocks, 256, 0, stream>>>(
                 (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, eps,
                 (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
-                write_kv ? (split_v ? 2 : 1) : 0, total_heads);
+                write_kv ? (split_v ? 2 : 1) : 0, total_heads, blocks, N);
         else
             qk_norm_rope_write_vec_kernel<<<blocks, 256, 0, stream>>>(
                 (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, rot,
