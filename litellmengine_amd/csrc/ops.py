@@ -402,7 +402,6 @@ class HipOps:
     force_separate_rope = False      # tests flip this to compare the fused decode step with its two halves
     # measured on MI355X: about one workgroup per CU and at least 8 32-key steps (two per
     # wavefront) per split are best; more splits cost more in partial results than they gain
-    DECODE_TARGET_BLOCKS = 256
     DECODE_MIN_STEPS_PER_SPLIT = 8
 
     PREFILL_MIN_STEPS_PER_SPLIT = 8
@@ -416,10 +415,17 @@ class HipOps:
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
         steps = (span + 31) // 32
         by_work = max(1, steps // self.PREFILL_MIN_STEPS_PER_SPLIT)
-        by_fill = max(1, self.DECODE_TARGET_BLOCKS // blocks)
+        by_fill = max(1, self.compute_units() // blocks)
         return int(min(by_work, by_fill, 64))
 
     _compute_units: dict = {}
+
+    def compute_units(self, device=None) -> int:
+        """CUs of `device` (the current one if not given), asked once per device."""
+        key = device.index if device is not None and device.index is not None else torch.cuda.current_device()
+        if key not in self._compute_units:
+            self._compute_units[key] = torch.cuda.get_device_properties(key).multi_processor_count
+        return self._compute_units[key]
 
     def prefill_form(self, num_seqs: int, num_kv_heads: int, group: int, head_dim: int, max_q_len: int,
                      max_kv_len: int, window: int, nsplit: int, device) -> int:
@@ -436,10 +442,7 @@ class HipOps:
             return 1
         if self.force_prefill_form:
             return self.force_prefill_form if head_dim == 128 or self.force_prefill_form < 3 else 2
-        key = device.index if device.index is not None else torch.cuda.current_device()
-        if key not in self._compute_units:
-            self._compute_units[key] = torch.cuda.get_device_properties(key).multi_processor_count
-        resident = 2 * self._compute_units[key]
+        resident = 2 * self.compute_units(device)
         rows = max_q_len * group
         low = -(-rows // 64) * num_kv_heads * max(1, num_seqs) * max(1, nsplit)
         if low <= resident:
@@ -453,7 +456,7 @@ class HipOps:
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
         steps = (span + 15) // 16
         by_work = max(1, steps // 16)
-        by_fill = max(1, (2 * self.DECODE_TARGET_BLOCKS) // max(1, num_seqs * num_kv_heads * row_blocks))
+        by_fill = max(1, (2 * self.compute_units()) // max(1, num_seqs * num_kv_heads * row_blocks))
         return int(min(by_work, by_fill, 64))
 
     def decode_splits(self, num_seqs: int, num_kv_heads: int, max_kv_len: int, window: int) -> int:
@@ -462,7 +465,7 @@ class HipOps:
         span = min(max_kv_len, window + 32) if window else max_kv_len
         steps = (span + 31) // 32 + (1 if window else 0)
         by_work = max(1, steps // self.DECODE_MIN_STEPS_PER_SPLIT)
-        by_fill = max(1, self.DECODE_TARGET_BLOCKS // max(1, num_seqs * num_kv_heads))
+        by_fill = max(1, self.compute_units() // max(1, num_seqs * num_kv_heads))
         return int(min(by_work, by_fill, 64))
 
     # -- feed-forward --------------------------------------------------------------
