@@ -61,16 +61,19 @@ __device__ __forceinline__ float4 load_weight4(const void* w, int i, int dtype) 
 // The same sums in one pass for rows of up to 256 * 4 * NORM_CHUNKS elements (a multiple of 4):
 // every thread keeps its part of the row in registers between the sum and the scaling.
 #define NORM_CHUNKS 8
-template <typename T>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ hidden, const T* __restrict__ delta,
+// `delta` may come as `slices` partial sums of type TD, `slice_stride` elements apart (a product
+// over slices of K leaves them so): they are added in slice order.
+template <typename T, typename TD = T>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ hidden, const TD* __restrict__ delta,
                                                               const int32_t* __restrict__ rows,
                                                               const void* __restrict__ weight, int weight_dtype,
-                                                              T* __restrict__ out, int H, float eps) {
+                                                              T* __restrict__ out, int H, float eps, int slices = 1,
+                                                              int64_t slice_stride = 0) {
     __shared__ float red[16];
     const int64_t r = blockIdx.x;
     const int64_t row = rows ? (int64_t)rows[r] : r;
     float* h = hidden + row * H;
-    const T* dl = delta ? delta + row * H : nullptr;
+    const TD* dl = delta ? delta + row * H : nullptr;
     float4 v[NORM_CHUNKS], wv[NORM_CHUNKS];
     float ss = 0.f;
 #pragma unroll
@@ -84,7 +87,14 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         if (i < H) {
             float4 x = *(const float4*)(h + i);
             if (dl) {
-                const float4 d = Quad<T>::load(dl + i);
+                float4 d = Quad<TD>::load(dl + i);
+                for (int sl = 1; sl < slices; ++sl) {
+                    const float4 e = Quad<TD>::load(dl + sl * slice_stride + i);
+                    d.x += e.x;
+                    d.y += e.y;
+                    d.z += e.z;
+                    d.w += e.w;
+                }
                 x.x += d.x;
                 x.y += d.y;
                 x.z += d.z;
@@ -107,6 +117,24 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
                                               v[k].w * inv * w.w));
         }
     }
+}
+
+// hidden += sums[0] + sums[1] + ... (float32 [slices][N][H], rows of hidden and of a slice alike), then
+// the norm as lle_add_rmsnorm; H a multiple of 4 up to 256 * 4 * NORM_CHUNKS
+extern "C" int lle_add_rmsnorm_sums(void* hidden, const void* sums, int slices, int64_t slice_stride, const void* rows,
+                                    const void* weight, int weight_dtype, void* out, int R, int H, float eps, int dtype,
+                                    hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (H % 4 != 0 || H > 256 * 4 * NORM_CHUNKS || slices < 1 || !sums) return (int)hipErrorInvalidValue;
+    if (dtype == LLE_F32)
+        add_rmsnorm_vec_kernel<float, float><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
+                                                                     (const int32_t*)rows, weight, weight_dtype,
+                                                                     (float*)out, H, eps, slices, slice_stride);
+    else
+        add_rmsnorm_vec_kernel<bf16_t, float><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
+                                                                      (const int32_t*)rows, weight, weight_dtype,
+                                                                      (bf16_t*)out, H, eps, slices, slice_stride);
+    LLE_RETURN_LAUNCH_STATUS();
 }
 
 extern "C" int lle_add_rmsnorm(void* hidden, const void* delta, const void* rows, const void* weight,

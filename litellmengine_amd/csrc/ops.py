@@ -91,14 +91,20 @@ class HipOps:
 
     # -- norms ---------------------------------------------------------------
     def add_rmsnorm(self, hidden, delta, weight, eps: float, out_dtype, rows=None) -> torch.Tensor:
-        """hidden float32 [N, H] (+ delta [N, H] of out_dtype) -> norm * weight, out_dtype.
+        """hidden float32 [N, H] (+ delta [N, H] of out_dtype, or float32 partial sums
+        [slices, N, H] that are added in slice order) -> norm * weight, out_dtype.
         Without `rows` the sum is written back to `hidden` and every row is normed;
         with `rows` (int32 [R]) only those rows are read and nothing is written back."""
         _dev(hidden, "hidden", torch.float32)
         _dev(weight, "norm weight")
         N, H = hidden.shape
         _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
-        if delta is not None:
+        sums = delta is not None and delta.dim() == 3  # partial sums of a product taken in slices of K
+        if sums:
+            _dev(delta, "partial sums", torch.float32)
+            _need(delta.shape[1:] == hidden.shape and H % 4 == 0 and H <= 8192,
+                  f"partial sums {list(delta.shape)} do not fit the residual stream {list(hidden.shape)}")
+        elif delta is not None:
             _dev(delta, "delta", out_dtype)
             _need(delta.shape == hidden.shape, "delta must have the shape of hidden")
         if rows is not None:
@@ -107,6 +113,11 @@ class HipOps:
         else:
             R = N
         out = torch.empty((R, H), dtype=out_dtype, device=hidden.device)
+        if sums:
+            self._run("norm", "lle_add_rmsnorm_sums", [_P, _P, _I, _L, _P, _P, _I, _P, _I, _I, _F, _I, _P],
+                      _ptr(hidden), _ptr(delta), delta.shape[0], delta.stride(0), _ptr(rows), _ptr(weight),
+                      dtype_code(weight.dtype), _ptr(out), R, H, float(eps), dtype_code(out_dtype))
+            return out
         self._run("norm", "lle_add_rmsnorm", [_P, _P, _P, _P, _I, _P, _I, _I, _F, _I, _P],
                   _ptr(hidden), _ptr(delta), _ptr(rows), _ptr(weight), dtype_code(weight.dtype), _ptr(out),
                   R, H, float(eps), dtype_code(out_dtype))
@@ -173,8 +184,9 @@ class HipOps:
                   _ptr(xw), _ptr(sums), M, N, K)
         return Prenormed(xw, sums, fold.eps)
 
-    def linear(self, x, weight, out_dtype=None, fold=None):
-        """x [M, K] . weight [N, K]^T -> [M, N].  float32 operands take a true 32-bit
+    def linear(self, x, weight, out_dtype=None, fold=None, sums_ok=False):
+        """x [M, K] . weight [N, K]^T -> [M, N].  With `sums_ok` the caller takes the result also as
+        float32 partial sums [slices, M, N] (what add_rmsnorm adds into the residual stream).  float32 operands take a true 32-bit
         product: few rows the weight-streaming kernel, more rows a tiled kernel, both
         with the float32 matrix instruction; the plain-FMA kernel where K is no multiple of 4.  bfloat16 operands: few rows take the
         weight-streaming matrix-core kernel, more rows the library product; both
@@ -190,6 +202,10 @@ class HipOps:
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
         out_dtype = out_dtype or x.dtype
         if x.dtype == torch.bfloat16:
+            if sums_ok and out_dtype == torch.bfloat16:
+                slices = self.slices_for(M, N, K)
+                if slices:
+                    return self.linear_slices(x, weight, slices)
             skinny = K % 8 == 0 and not self.force_library_gemm and (
                 M <= self.SKINNY_MAX_ROWS or (M <= 16 and N * K <= self.SKINNY_SMALL_WEIGHT))
             if skinny:
@@ -213,6 +229,43 @@ class HipOps:
             return out
         self._run("gemm", "lle_gemm_nt_simt", [_P, _P, _P, _I, _I, _I, _L, _L, _L, _I, _I, _P],
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
+        return out
+
+    SLICED_MIN_ROWS, SLICED_MAX_ROWS = 17, 64
+    SLICED_UNIT = 1024  # columns of K that a slice is a multiple of (lle_gemm_mid_slices_unit)
+
+    def slices_for(self, M: int, N: int, K: int) -> int:
+        """In how many slices of K the product of 17 to 64 rows with a weight [N, K] is taken
+        (see linear_slices), or 0 where the library product stays: the workgroups, N / 64 x slices,
+        have to fill the CUs in whole rounds (at least 0.85 of them), which weights with few rows
+        per CU do (o_proj, down_proj) and wide ones need no slices for."""
+        if not (self.SLICED_MIN_ROWS <= M <= self.SLICED_MAX_ROWS) or N % 64 != 0 or self.force_library_gemm:
+            return 0
+        units = self.compute_units()
+        if N // 64 > units // 2:  # enough rows for the library's own tiles
+            return 0
+        for slices in (2, 3, 4, 6, 8):
+            if K % (self.SLICED_UNIT * slices) != 0:
+                continue
+            groups = (N // 64) * slices
+            rounds = -(-groups // units)
+            if groups >= 0.85 * rounds * units:
+                return slices
+        return 0
+
+    def linear_slices(self, x, weight, slices: int) -> torch.Tensor:
+        """x [M, K] . weight [N, K]^T as float32 partial sums over `slices` equal parts of K:
+        [slices, M, N], to be added up by the reader in slice order (M <= 64)."""
+        _dev(x, "x", torch.bfloat16)
+        _dev(weight, "weight", torch.bfloat16)
+        M, K = x.shape
+        N = weight.shape[0]
+        _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
+        _need(0 < M <= 64 and N % 64 == 0 and slices > 0 and K % (self.SLICED_UNIT * slices) == 0,
+              f"no product in {slices} slices for [{M}, {K}] x [{N}, {K}]")
+        out = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+        self._run("gemm", "lle_gemm_mid_slices_bf16", [_P, _P, _P, _I, _I, _I, _I, _P], _ptr(x), _ptr(weight), _ptr(out),
+                  M, N, K, slices)
         return out
 
     # measured on MI355X: the weight-streaming kernels (with the norm folded into them) win up to 16

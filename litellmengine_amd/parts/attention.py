@@ -54,7 +54,7 @@ class PagedAttention(Mixer):
             hidden_size,
             [num_q_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
         )
-        self.o = Linear([prefix + "o_proj.weight"], num_q_heads * head_dim, [hidden_size])
+        self.o = Linear([prefix + "o_proj.weight"], num_q_heads * head_dim, [hidden_size], to_residual=True)
         self.q_norm_w = None
         self.k_norm_w = None
 

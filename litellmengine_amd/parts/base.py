@@ -127,7 +127,10 @@ class Prenormed:
 class Norm(Part):
     """forward(hidden, delta) adds `delta` (or nothing) into the 32-bit residual
     stream `hidden` in place and returns the normed rows in the activation type;
-    with `rows` only those rows are read and `hidden` is left alone.
+    with `rows` only those rows are read and `hidden` is left alone.  `delta` is
+    [N, hidden] in the activation type, or float32 partial sums [slices, N, hidden]
+    that are to be added in slice order (a Linear made with `to_residual` may leave
+    them so; `delta.sum(0)` is the plain way to take them).
 
     fold(hidden) may return a NormFold when the step is small enough that the
     products on both sides of the norm can do its work (None: call forward)."""

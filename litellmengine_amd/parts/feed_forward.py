@@ -19,7 +19,7 @@ class GatedMLP(FeedForward):
         self.gate_up = Linear(
             [prefix + "gate_proj.weight", prefix + "up_proj.weight"], hidden_size, [intermediate_size] * 2
         )
-        self.down = Linear([prefix + "down_proj.weight"], intermediate_size, [hidden_size])
+        self.down = Linear([prefix + "down_proj.weight"], intermediate_size, [hidden_size], to_residual=True)
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         return {**self.gate_up.tensor_specs(), **self.down.tensor_specs()}

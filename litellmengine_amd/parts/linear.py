@@ -13,11 +13,16 @@ from .base import BuildContext, Part
 
 
 class Linear(Part):
-    def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int], optional: bool = False):
+    def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int], optional: bool = False,
+                 to_residual: bool = False):
+        """`to_residual`: the result is a delta of the residual stream and goes nowhere but into
+        Norm.forward(hidden, delta); it may then come as float32 partial sums [slices, N, out]
+        (a product taken in slices of `in`), which that call adds up."""
         self.names = list(names)
         self.in_features = in_features
         self.out_features = list(out_features)
         self.optional = optional
+        self.to_residual = to_residual
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -40,5 +45,7 @@ class Linear(Part):
         """`x` may be a parts.base.Prenormed; with `fold` (a parts.base.NormFold) the result
         is added into the residual stream and comes back as the Prenormed of that norm."""
         if fold is None:
+            if self.to_residual and out_dtype is None and hasattr(self.ctx.ops, "slices_for"):
+                return self.ctx.ops.linear(x, self.weight, out_dtype, sums_ok=True)
             return self.ctx.ops.linear(x, self.weight, out_dtype)
         return self.ctx.ops.linear(x, self.weight, out_dtype, fold=fold)

@@ -149,6 +149,59 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         assert (got.double() - ref.double()).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("N,K,slices", [(4096, 4096, 4), (4096, 12288, 4), (320, 2048, 2), (64, 1024, 1), (128, 3072, 3)])
+def test_product_in_slices_of_k(M, N, K, slices):
+    """The product of 17 to 64 rows taken in slices of K: the float32 partial sums add up to the
+    float64 product, each slice is the product over its own columns, and the residual add + norm
+    that reads them gives what it gives for the summed delta.  W is made of rows that tell their
+    own number and X of rows that tell theirs, so a tile written to the wrong place shows."""
+    o = ops()
+    x = rnd((M, K), torch.bfloat16, 61)
+    w = rnd((N, K), torch.bfloat16, 62, 0.05)
+    w[:, 0] = (torch.arange(N) % 64).to(torch.bfloat16) / 16
+    x[:, 1] = (torch.arange(M) % 16).to(torch.bfloat16) / 8
+    got = o.linear_slices(x, w, slices)
+    assert got.shape == (slices, M, N) and got.dtype == torch.float32
+    part = K // slices
+    for s in range(slices):
+        want = x[:, s * part:(s + 1) * part].double() @ w[:, s * part:(s + 1) * part].double().t()
+        assert (got[s].double() - want).abs().max() < 2e-4 * max(1.0, want.abs().max().item()), s
+    if N % 4 == 0 and N <= 8192:
+        hidden = rnd((M, N), torch.float32, 63, 1.5)
+        nw = (1 + 0.3 * rnd((N,), torch.float32, 64)).to(torch.bfloat16)
+        h_ref = hidden.clone()
+        want = REF.add_rmsnorm(h_ref, got, nw, 1e-6, torch.bfloat16)
+        h_got = hidden.clone()
+        out = o.add_rmsnorm(h_got, got, nw, 1e-6, torch.bfloat16)
+        assert (h_got.double() - h_ref.double()).abs().max() < 1e-5 * max(1.0, h_ref.abs().max().item())
+        assert (out.double() - want.double()).abs().max() < 2e-2
+        rows = torch.tensor([M - 1, 0, 5], dtype=torch.int32, device="cuda")
+        h_keep = hidden.clone()
+        picked = o.add_rmsnorm(h_keep, got, nw, 1e-6, torch.bfloat16, rows=rows)
+        assert torch.equal(h_keep, hidden)  # with rows nothing is written back
+        assert (picked.double() - want[rows.long()].double()).abs().max() < 2e-2
+
+
+def test_which_products_are_taken_in_slices():
+    """The choice is made from the sizes and the CU count: few rows per CU (o_proj, down_proj of the
+    8B sizes) in whole rounds of workgroups; not below 17 or above 64 rows, not for wide weights,
+    not where no slice count fills the CUs; and the engine's Linear asks only for deltas of the
+    residual stream."""
+    o = ops()
+    units = o.compute_units()
+    n = 16 * units  # 16 rows a CU
+    assert o.slices_for(64, n, 4096) == 4 and o.slices_for(17, n, 12288) == 4
+    assert o.slices_for(16, n, 4096) == 0 and o.slices_for(65, n, 4096) == 0
+    assert o.slices_for(64, 64 * units, 4096) == 0      # wide: rows enough for every CU
+    assert o.slices_for(64, n + 8, 4096) == 0           # no multiple of 64 rows
+    assert o.slices_for(64, n, 4096 + 256) == 0         # no whole slices
+    x = rnd((40, 4096), torch.bfloat16, 65)
+    w = rnd((n, 4096), torch.bfloat16, 66, 0.05)
+    assert o.linear(x, w).shape == (40, n)                       # a caller that said nothing gets the product
+    assert o.linear(x, w, sums_ok=True).shape == (4, 40, n)      # a delta of the residual stream may come in slices
+
+
 @pytest.mark.parametrize("K", [1024, 2048, 3072, 4096, 5120, 6144, 8192])
 @pytest.mark.parametrize("M", [1, 7, 16])
 def test_streaming_products_at_every_width(M, K):

@@ -27,6 +27,8 @@ class TorchOps:
         return table[ids.long()].to(torch.float32)
 
     def add_rmsnorm(self, hidden, delta, weight, eps, out_dtype, rows=None):
+        if delta is not None and delta.dim() == 3:  # partial sums of a product taken in slices
+            delta = delta.to(self.cd).sum(0)
         if rows is None:
             if delta is not None:
                 hidden += delta.to(hidden.dtype)
