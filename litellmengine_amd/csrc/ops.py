@@ -486,9 +486,9 @@ class HipOps:
           1: four wavefronts of one 16-row tile each (64 rows a workgroup),
           2: four wavefronts of two tiles each (128 rows; every operand read from LDS serves both tiles),
           3: eight wavefronts of one tile each (128 rows; four wavefronts a SIMD; heads of 128 only).
-        The low form when its workgroups all fit the chip at once (a short portion); else the tall
-        ones, which share a pass over the keys between more rows: form 3 at heads of 128, form 2
-        below.  Measured on MI355X at heads of 128 (forms 1 / 2 / 3): 2048 tokens from an empty cache
+        The low form when its workgroups all fit the chip at once (a short portion; at heads of 128
+        only one prompt from an empty cache); else the tall ones, which share a pass over the keys between more
+        rows: form 3 at heads of 128, form 2 below.  Measured on MI355X at heads of 128 (forms 1 / 2 / 3): 2048 tokens from an empty cache
         60 / 65 / 57 us, 2048 tokens after 2048 keys 148 / 128 / 118 us, 49 tokens after 2048 keys
         17 / 21 / 19 us."""
         if head_dim > 128:
@@ -498,9 +498,11 @@ class HipOps:
         resident = 2 * self.compute_units(device)
         rows = max_q_len * group
         low = -(-rows // 64) * num_kv_heads * max(1, num_seqs) * max(1, nsplit)
-        if low <= resident:
-            return 1
-        return 3 if head_dim == 128 else 2
+        if head_dim == 128:
+            # (measured: form 3 wins by 5-15 % whenever there is a past or more than one request; one
+            # prompt from an empty cache is up to 10 % faster in the low form while that fits the chip at once)
+            return 1 if low <= resident and max_kv_len <= max_q_len and num_seqs <= 1 else 3
+        return 1 if low <= resident else 2
 
     def f32_attention_splits(self, num_seqs: int, num_kv_heads: int, row_blocks: int, max_q_len: int,
                              max_kv_len: int, window: int) -> int:
