@@ -43,10 +43,27 @@ def _need(cond: bool, msg: str) -> None:
 
 
 def _dev(t: torch.Tensor, name: str, dtype=None) -> None:
-    _need(t.is_cuda, f"{name} must live on the GPU")
-    _need(t.is_contiguous(), f"{name} must be contiguous")
-    if dtype is not None:
-        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+    # (on every operand of every launch: the messages are made only when they are needed)
+    if not t.is_cuda:
+        raise KernelError(f"{name} must live on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, is {t.dtype}")
+
+
+# the current stream's handle without the Stream object around it (a launch is a few microseconds
+# of Python as it is; torch.cuda.current_stream() alone costs as much again)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def _stream_handle() -> int:
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 class HipOps:
@@ -72,7 +89,7 @@ class HipOps:
 
     def _run(self, lib: str, name: str, argtypes, *args):
         fn = self._get(lib, name, argtypes)
-        code = fn(*args, torch.cuda.current_stream().cuda_stream)
+        code = fn(*args, _stream_handle())
         if code != 0:
             msg = build.load_library(lib).lle_error_string(code).decode()
             raise KernelError(f"{name} failed to launch: {msg} (hip error {code})")
