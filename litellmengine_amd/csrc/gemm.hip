@@ -405,7 +405,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 }
 
 // ---------------------------------------------------------------------------------
-// 17 to 64 rows of X against a weight with few rows per CU (N about 16 rows a CU: o_proj,
+// 17 to 128 rows of X against a weight with few rows per CU (N about 16 rows a CU: o_proj,
 // down_proj): the product in SLICES of K.  With one 16-row tile of W per workgroup every
 // workgroup reads all of X (at 64 rows four times the bytes of its share of W, through L2), and
 // taller tiles leave CUs without work: so a workgroup takes 64 rows of W and one of `slices`
@@ -420,20 +420,24 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE, (MT == 1 && !GATED) ? 8 : 4) vo
 //     sixteen lanes that a 16-byte LDS read serves in a cycle hit sixteen different columns of
 //     the banks, and every wavefront multiplies its W operands with every 16-row tile of it;
 //   * at the end the four steps of a tile are added up in LDS.
-// Measured on MI355X at 64 rows against the library: o_proj sizes (4096 x 4096) 11.7 against
-// 15.0 us, down_proj sizes (4096 x 12288) 29.5 against 38.7 us; a CU takes in about 29 GB/s of
-// W and X together whatever the depth of the loads on their way.
+// Measured on MI355X against the library: o_proj sizes (4096 x 4096) 11.7 against 15.0 us at
+// 64 rows and 15.8 against 24.3 at 128, down_proj sizes (4096 x 12288) 29.5 against 38.7 us and
+// 37.2 against 67.6; a CU takes in about 29 GB/s of W and X together whatever the depth of the
+// loads on their way, and at 128 rows a workgroup reads twice as much X as W.
 // ---------------------------------------------------------------------------------
 #define MID_ROWS 64    // rows of W per workgroup
 #define MID_STEPS 4    // 64-element steps of K per stage: 4 x MID_STEPS wavefronts a workgroup
-#define MID_BUFFERS 4  // register sets: stages on their way from memory, plus the one that is multiplied
+#define MID_UNIT_STAGES 4  // a slice of K is a whole number of these many stages (the register sets divide it)
 #define MID_STAGE (64 * MID_STEPS)  // columns of K per stage
 // The XOR of a 16-byte piece index in row r of a 16-row tile of X.  Lanes (c, r) read the pieces
 // 2 c and 2 c + 1 of a step; a cycle serves c0 with r / 4 in {0, 3} and c0 + 1 with r / 4 in
 // {1, 2} (or the other way round), whose pieces differ in bit 1: r % 4 goes to bits 2-3 and
 // r / 8 to bit 0, which makes the sixteen columns different.
 #define MID_SWIZZLE(r) ((((r) & 3) << 2) | (((r) >> 3) & 1))
-template <int M_TILES>
+// BUFFERS: register sets, i.e. the stages on their way from memory plus the one that is multiplied
+// (four up to 64 rows of X; two at 128 rows, where a stage of X is four loads a thread and the
+// sixteen wavefronts of a workgroup have 128 registers a lane each; one to four measured the same).
+template <int M_TILES, int BUFFERS>
 __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kernel(const bf16_t* __restrict__ X,
                                                                                   const bf16_t* __restrict__ W,
                                                                                   float* __restrict__ out, int M, int N,
@@ -464,7 +468,7 @@ __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kern
         xsrc[i] = X + (int64_t)min(m, M - 1) * K + k_begin + 8 * p;
         xdst[i] = m * MID_STAGE + 8 * (p ^ MID_SWIZZLE(m % 16));
     }
-    gbf16x8 w0[MID_BUFFERS], w1[MID_BUFFERS], xr[MID_BUFFERS][XL];
+    gbf16x8 w0[BUFFERS], w1[BUFFERS], xr[BUFFERS][XL];
     auto issue = [&](int st, auto buf_c) {
         constexpr int buf = decltype(buf_c)::value;
         w0[buf] = *(const gbf16x8*)(wp + st * MID_STAGE);
@@ -478,7 +482,7 @@ __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kern
     const int sw = MID_SWIZZLE(r16);
     const int piece0 = 8 * step + 2 * c;  // logical pieces 2 c and 2 c + 1 of the wavefront's step
     const int x_read0 = r16 * MID_STAGE + 8 * (piece0 ^ sw), x_read1 = r16 * MID_STAGE + 8 * ((piece0 + 1) ^ sw);
-    // Stage st waits in register set st % MID_BUFFERS (MID_BUFFERS - 1 stages are on their way from
+    // Stage st waits in register set st % BUFFERS (BUFFERS - 1 stages are on their way from
     // memory while one is multiplied) and is multiplied from LDS buffer st % 2.
     auto run_stage = [&](int st, auto buf_c) {
         constexpr int buf = decltype(buf_c)::value;
@@ -491,7 +495,7 @@ __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kern
         __builtin_amdgcn_s_barrier();  // all of stage st is in LDS, and nobody reads stage st - 1 any more
         // (asked for under no condition, past the end the last stage again: where paths meet the
         // compiler would wait for every load that one of them may have issued)
-        issue(min(st + MID_BUFFERS - 1, stages - 1), std::integral_constant<int, (buf + MID_BUFFERS - 1) % MID_BUFFERS>{});
+        issue(min(st + BUFFERS - 1, stages - 1), std::integral_constant<int, (buf + BUFFERS - 1) % BUFFERS>{});
 #pragma unroll
         for (int mt = 0; mt < M_TILES; ++mt) {
             const gbf16x8 x0 = *(const gbf16x8*)(xb + 16 * mt * MID_STAGE + x_read0);
@@ -500,13 +504,13 @@ __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kern
             acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[buf], x1, acc[mt], 0, 0, 0);
         }
     };
-    static_assert(MID_BUFFERS >= 2 && MID_BUFFERS <= 5, "register sets for the stages on their way");
-    // the number of stages is a multiple of MID_BUFFERS (the caller sees to it)
-#define MID_FOR_BUFFERS(F) F(0) F(1) F(2) F(3) F(4)
-#define MID_ISSUE_FIRST(B) if constexpr (B < MID_BUFFERS - 1) issue(min(B, stages - 1), std::integral_constant<int, B % MID_BUFFERS>{});
+    static_assert(BUFFERS >= 2 && BUFFERS <= 4 && MID_UNIT_STAGES % BUFFERS == 0, "register sets for the stages on their way");
+    // the number of stages is a multiple of MID_UNIT_STAGES, and so of BUFFERS (the caller sees to it)
+#define MID_FOR_BUFFERS(F) F(0) F(1) F(2) F(3)
+#define MID_ISSUE_FIRST(B) if constexpr (B < BUFFERS - 1) issue(min(B, stages - 1), std::integral_constant<int, B % BUFFERS>{});
     MID_FOR_BUFFERS(MID_ISSUE_FIRST)
-    for (int st = 0; st < stages; st += MID_BUFFERS) {
-#define MID_RUN(B) if constexpr (B < MID_BUFFERS) run_stage(st + B, std::integral_constant<int, B % MID_BUFFERS>{});
+    for (int st = 0; st < stages; st += BUFFERS) {
+#define MID_RUN(B) if constexpr (B < BUFFERS) run_stage(st + B, std::integral_constant<int, B % BUFFERS>{});
         MID_FOR_BUFFERS(MID_RUN)
     }
 #undef MID_RUN
@@ -532,34 +536,39 @@ __global__ __launch_bounds__(4 * MID_STEPS * LLE_WAVE) void gemm_mid_slices_kern
     }
 }
 
-// out [slices][M][N] float32; M <= 64, N a multiple of 64, K a multiple of slices x 4 stages of 256 columns
-extern "C" int lle_gemm_mid_slices_unit(void) { return MID_STAGE * MID_BUFFERS; }
+// out [slices][M][N] float32; M <= 128, N a multiple of 64, K a multiple of slices x 4 stages of 256 columns
+extern "C" int lle_gemm_mid_slices_unit(void) { return MID_STAGE * MID_UNIT_STAGES; }
+extern "C" int lle_gemm_mid_slices_max_rows(void) { return 128; }
 
 extern "C" int lle_gemm_mid_slices_bf16(const void* X, const void* W, void* out, int M, int N, int K, int slices,
                                         hipStream_t stream) {
-    if (M <= 0 || M > 64 || N % MID_ROWS != 0 || slices <= 0 || slices > 65535 || K % (MID_STAGE * MID_BUFFERS * slices) != 0)
+    if (M <= 0 || M > 128 || N % MID_ROWS != 0 || slices <= 0 || slices > 65535 || K % (MID_STAGE * MID_UNIT_STAGES * slices) != 0)
         return (int)hipErrorInvalidValue;
     const dim3 grid(N / MID_ROWS, slices);
     const int stages = K / (MID_STAGE * slices);
-#define LLE_MID_LAUNCH(T)                                                                                             \
+#define LLE_MID_LAUNCH(T, B)                                                                                          \
     {                                                                                                                 \
         constexpr size_t tiles = (size_t)2 * 16 * T * MID_STAGE * sizeof(bf16_t);                           \
         constexpr size_t sums = (size_t)4 * MID_STEPS * T * 16 * 17 * sizeof(float);                                  \
         constexpr size_t lds = tiles > sums ? tiles : sums;                                                           \
         static bool ready = false; /* more than 64 KB of LDS has to be asked for once */                              \
         if (!ready) {                                                                                                 \
-            if (hipFuncSetAttribute((const void*)gemm_mid_slices_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+            if (hipFuncSetAttribute((const void*)gemm_mid_slices_kernel<T, B>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                     (int)lds) != hipSuccess)                                                          \
                 return (int)hipGetLastError();                                                                        \
             ready = true;                                                                                             \
         }                                                                                                             \
-        gemm_mid_slices_kernel<T><<<grid, 4 * MID_STEPS * LLE_WAVE, lds, stream>>>(                                    \
+        gemm_mid_slices_kernel<T, B><<<grid, 4 * MID_STEPS * LLE_WAVE, lds, stream>>>(                                    \
             (const bf16_t*)X, (const bf16_t*)W, (float*)out, M, N, K, stages);                                        \
     }
     if (M <= 32)
-        LLE_MID_LAUNCH(2)
+        LLE_MID_LAUNCH(2, 4)
+    else if (M <= 64)
+        LLE_MID_LAUNCH(4, 4)
+    else if (M <= 96)
+        LLE_MID_LAUNCH(6, 2)
     else
-        LLE_MID_LAUNCH(4)
+        LLE_MID_LAUNCH(8, 2)
 #undef LLE_MID_LAUNCH
     LLE_RETURN_LAUNCH_STATUS();
 }

@@ -248,11 +248,11 @@ class HipOps:
                   _ptr(x), _ptr(weight), _ptr(out), M, N, K, K, K, N, dtype_code(x.dtype), dtype_code(out_dtype))
         return out
 
-    SLICED_MIN_ROWS, SLICED_MAX_ROWS = 17, 64
+    SLICED_MIN_ROWS, SLICED_MAX_ROWS = 17, 128  # (lle_gemm_mid_slices_max_rows)
     SLICED_UNIT = 1024  # columns of K that a slice is a multiple of (lle_gemm_mid_slices_unit)
 
     def slices_for(self, M: int, N: int, K: int) -> int:
-        """In how many slices of K the product of 17 to 64 rows with a weight [N, K] is taken
+        """In how many slices of K the product of 17 to 128 rows with a weight [N, K] is taken
         (see linear_slices), or 0 where the library product stays: the workgroups, N / 64 x slices,
         have to fill the CUs in whole rounds (at least 0.85 of them), which weights with few rows
         per CU do (o_proj, down_proj) and wide ones need no slices for."""
@@ -272,13 +272,13 @@ class HipOps:
 
     def linear_slices(self, x, weight, slices: int) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T as float32 partial sums over `slices` equal parts of K:
-        [slices, M, N], to be added up by the reader in slice order (M <= 64)."""
+        [slices, M, N], to be added up by the reader in slice order (M <= 128)."""
         _dev(x, "x", torch.bfloat16)
         _dev(weight, "weight", torch.bfloat16)
         M, K = x.shape
         N = weight.shape[0]
         _need(weight.shape[1] == K, f"weight [{N}, {weight.shape[1]}] does not fit x [{M}, {K}]")
-        _need(0 < M <= 64 and N % 64 == 0 and slices > 0 and K % (self.SLICED_UNIT * slices) == 0,
+        _need(0 < M <= self.SLICED_MAX_ROWS and N % 64 == 0 and slices > 0 and K % (self.SLICED_UNIT * slices) == 0,
               f"no product in {slices} slices for [{M}, {K}] x [{N}, {K}]")
         out = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
         self._run("gemm", "lle_gemm_mid_slices_bf16", [_P, _P, _P, _I, _I, _I, _I, _P], _ptr(x), _ptr(weight), _ptr(out),

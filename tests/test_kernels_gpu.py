@@ -149,10 +149,10 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
         assert (got.double() - ref.double()).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
 
 
-@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64, 65, 81, 96, 97, 128])
 @pytest.mark.parametrize("N,K,slices", [(4096, 4096, 4), (4096, 12288, 4), (320, 2048, 2), (64, 1024, 1), (128, 3072, 3)])
 def test_product_in_slices_of_k(M, N, K, slices):
-    """The product of 17 to 64 rows taken in slices of K: the float32 partial sums add up to the
+    """The product of 17 to 128 rows taken in slices of K: the float32 partial sums add up to the
     float64 product, each slice is the product over its own columns, and the residual add + norm
     that reads them gives what it gives for the summed delta.  W is made of rows that tell their
     own number and X of rows that tell theirs, so a tile written to the wrong place shows."""
@@ -185,14 +185,14 @@ def test_product_in_slices_of_k(M, N, K, slices):
 
 def test_which_products_are_taken_in_slices():
     """The choice is made from the sizes and the CU count: few rows per CU (o_proj, down_proj of the
-    8B sizes) in whole rounds of workgroups; not below 17 or above 64 rows, not for wide weights,
+    8B sizes) in whole rounds of workgroups; not below 17 or above 128 rows, not for wide weights,
     not where no slice count fills the CUs; and the engine's Linear asks only for deltas of the
     residual stream."""
     o = ops()
     units = o.compute_units()
     n = 16 * units  # 16 rows a CU
     assert o.slices_for(64, n, 4096) == 4 and o.slices_for(17, n, 12288) == 4
-    assert o.slices_for(16, n, 4096) == 0 and o.slices_for(65, n, 4096) == 0
+    assert o.slices_for(128, n, 4096) == 4 and o.slices_for(16, n, 4096) == 0 and o.slices_for(129, n, 4096) == 0
     assert o.slices_for(64, 64 * units, 4096) == 0      # wide: rows enough for every CU
     assert o.slices_for(64, n + 8, 4096) == 0           # no multiple of 64 rows
     assert o.slices_for(64, n, 4096 + 256) == 0         # no whole slices
