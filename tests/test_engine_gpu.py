@@ -124,12 +124,13 @@ def test_qwen3_8b_layer_sizes(tmp_path):
     d = str(tmp_path / "m8b")
     write_model_dir(cfg, d, 3, torch.bfloat16)
     pcfg, w = plain.read_model_dir(d, dtype=torch.float32)
-    tokens = random_tokens(70, cfg.vocab_size, 5)
+    tokens = random_tokens(120, cfg.vocab_size, 5)
     want = plain.model_logits_fast(tokens, w, pcfg).double()
     scale = max(1.0, want.abs().max().item())
     for dtype, tol in (("float32", 2e-5), ("bfloat16", 4e-2)):  # the oracle itself is float32 here
         runner = make_runner(d, dtype, 16, 8)
-        for cuts in ([70], [38] + [1] * 32, [2, 17, 3, 30, 18]):
+        # (120, 88 and 68 rows: o_proj and down_proj in slices of K with eight, six and six tiles of rows)
+        for cuts in ([120], [88] + [1] * 32, [2, 17, 3, 30, 68]):
             got = run_cut(runner, tokens, cuts)
             err = (got.double() - want).abs().max().item() / scale
             assert err < tol, (dtype, cuts, err)
