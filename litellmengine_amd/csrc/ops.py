@@ -483,9 +483,10 @@ class HipOps:
         every row sees count (the past; a prompt from an empty cache is never split: measured
         twice as slow at 512 tokens).  A split keeps at least 8 steps of 32 keys while the row
         blocks fill less than half the CUs and 32 otherwise, the splits fill the CUs once, and
-        twice where every split still keeps 32 steps (measured: 128 tokens after 1 k keys 26 -> 20 us
-        with 4 splits, 512 tokens after 16 k keys 289 -> 149 us with 4, 512 tokens after 1 k keys
-        best unsplit)."""
+        twice where every split still keeps 32 steps and the row blocks alone fill at most half the
+        CUs (measured: 128 tokens after 1 k keys 26 -> 20 us with 4 splits, 512 tokens after 16 k
+        keys 289 -> 149 us with 4, 512 tokens after 1 k keys best unsplit; row blocks that fill the
+        CUs by themselves are never split: 2048 tokens after 2048 keys 115 us unsplit, 151 in two)."""
         units = self.compute_units()
         rows_per_block = 128 if head_dim <= 128 else 64
         blocks = ((max_q_len * group + rows_per_block - 1) // rows_per_block) * num_kv_heads * max(1, num_seqs)
@@ -496,7 +497,7 @@ class HipOps:
         by_work = max(1, steps // (self.PREFILL_MIN_STEPS_PER_SPLIT if 2 * blocks < units else 32))
         by_fill = max(1, units // blocks)
         splits = min(by_work, by_fill)
-        if splits == by_fill and steps // (2 * splits) >= 32:
+        if splits == by_fill and 2 * blocks <= units and steps // (2 * splits) >= 32:
             splits *= 2
         return int(min(splits, 64))
 

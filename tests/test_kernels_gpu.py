@@ -183,6 +183,22 @@ def test_product_in_slices_of_k(M, N, K, slices):
         assert (picked.double() - want[rows.long()].double()).abs().max() < 2e-2
 
 
+def test_key_splits_of_prompt_portions():
+    """The choice of key splits for prompt portions, from the sizes and the CU count: none from an
+    empty cache, none where the row blocks fill the CUs by themselves (a 2048-token portion of a
+    long prompt), several for a short portion after a long past."""
+    o = ops()
+    units = o.compute_units()
+    full = units // 8 * 128 // 4  # tokens whose row blocks (8 kv heads, groups of 4, 128 rows) fill the CUs once
+    assert o.prefill_splits(1, 8, 4, 128, 2048, 2048, 0) == 1
+    assert o.prefill_splits(1, 8, 4, 128, 2 * full, 2 * full + 2048, 0) == 1
+    assert o.prefill_splits(1, 8, 4, 128, full, full + 8192, 0) == 1
+    assert o.prefill_splits(1, 8, 4, 128, full // 2, full // 2 + 4096, 0) == 4
+    assert o.prefill_splits(1, 8, 4, 128, full // 2, full // 2 + 1024, 0) == 1
+    assert o.prefill_splits(1, 8, 4, 128, full // 8, full // 8 + 1024, 0) == 4
+    assert o.prefill_splits(1, 8, 4, 128, full // 8, full // 8 + 1024, 64) == 1  # a window of 64 keys
+
+
 def test_which_products_are_taken_in_slices():
     """The choice is made from the sizes and the CU count: few rows per CU (o_proj, down_proj of the
     8B sizes) in whole rounds of workgroups; not below 17 or above 128 rows, not for wide weights,
