@@ -483,10 +483,11 @@ class HipOps:
         every row sees count (the past; a prompt from an empty cache is never split: measured
         twice as slow at 512 tokens).  A split keeps at least 8 steps of 32 keys while the row
         blocks fill less than half the CUs and 32 otherwise, the splits fill the CUs once, and
-        twice where every split still keeps 32 steps and the row blocks alone fill at most half the
-        CUs (measured: 128 tokens after 1 k keys 26 -> 20 us with 4 splits, 512 tokens after 16 k
+        twice where every split still keeps 32 steps, at least two row blocks share the keys of a
+        head and the row blocks alone fill at most half the CUs (measured: 128 tokens after 1 k keys 26 -> 20 us with 4 splits, 512 tokens after 16 k
         keys 289 -> 149 us with 4, 512 tokens after 1 k keys best unsplit; row blocks that fill the
-        CUs by themselves are never split: 2048 tokens after 2048 keys 115 us unsplit, 151 in two)."""
+        CUs by themselves are never split: 2048 tokens after 2048 keys 115 us unsplit, 151 in two;
+        four requests of 32 tokens after 16 k keys 57 us in 8 splits, one workgroup a CU, 70 in 16)."""
         units = self.compute_units()
         rows_per_block = 128 if head_dim <= 128 else 64
         blocks = ((max_q_len * group + rows_per_block - 1) // rows_per_block) * num_kv_heads * max(1, num_seqs)
@@ -497,7 +498,8 @@ class HipOps:
         by_work = max(1, steps // (self.PREFILL_MIN_STEPS_PER_SPLIT if 2 * blocks < units else 32))
         by_fill = max(1, units // blocks)
         splits = min(by_work, by_fill)
-        if splits == by_fill and 2 * blocks <= units and steps // (2 * splits) >= 32:
+        shared_keys = max_q_len * group >= 2 * rows_per_block  # else the keys' way from memory bounds the launch
+        if splits == by_fill and 2 * blocks <= units and shared_keys and steps // (2 * splits) >= 32:
             splits *= 2
         return int(min(splits, 64))
 
@@ -517,7 +519,7 @@ class HipOps:
           2: four wavefronts of two tiles each (128 rows; every operand read from LDS serves both tiles),
           3: eight wavefronts of one tile each (128 rows; four wavefronts a SIMD; heads of 128 only).
         The low form when its workgroups all fit the chip at once (a short portion; at heads of 128
-        only one prompt from an empty cache); else the tall ones, which share a pass over the keys between more
+        at most one workgroup a CU, or one prompt from an empty cache); else the tall ones, which share a pass over the keys between more
         rows: form 3 at heads of 128, form 2 below.  Measured on MI355X at heads of 128 (forms 1 / 2 / 3): 2048 tokens from an empty cache
         60 / 65 / 57 us, 2048 tokens after 2048 keys 148 / 128 / 118 us, 49 tokens after 2048 keys
         17 / 21 / 19 us."""
@@ -529,9 +531,11 @@ class HipOps:
         rows = max_q_len * group
         low = -(-rows // 64) * num_kv_heads * max(1, num_seqs) * max(1, nsplit)
         if head_dim == 128:
-            # (measured: form 3 wins by 5-15 % whenever there is a past or more than one request; one
-            # prompt from an empty cache is up to 10 % faster in the low form while that fits the chip at once)
-            return 1 if low <= resident and max_kv_len <= max_q_len and num_seqs <= 1 else 3
+            # (measured: a launch of at most one low workgroup a CU is about 1 us, up to 10 %, faster in
+            # the low form, whatever its past and however many requests; so is one prompt from an empty
+            # cache while the low form fits the chip at once; else form 3 wins by 5-15 %)
+            units = resident // 2
+            return 1 if low <= units or (low <= resident and max_kv_len <= max_q_len and num_seqs <= 1) else 3
         return 1 if low <= resident else 2
 
     def f32_attention_splits(self, num_seqs: int, num_kv_heads: int, row_blocks: int, max_q_len: int,

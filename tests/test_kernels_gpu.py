@@ -197,6 +197,12 @@ def test_key_splits_of_prompt_portions():
     assert o.prefill_splits(1, 8, 4, 128, full // 2, full // 2 + 1024, 0) == 1
     assert o.prefill_splits(1, 8, 4, 128, full // 8, full // 8 + 1024, 0) == 4
     assert o.prefill_splits(1, 8, 4, 128, full // 8, full // 8 + 1024, 64) == 1  # a window of 64 keys
+    # one row block a head (the keys come from memory once, one workgroup a CU is best) against sixteen
+    assert o.prefill_splits(4, 8, 4, 128, 32, 32 + 16384, 0) == units // 32
+    assert o.prefill_splits(1, 8, 4, 128, full // 2, full // 2 + 16384, 0) == 4
+    # the low workgroup shape for a launch of at most one workgroup a CU, whatever its past
+    assert o.prefill_form(2, 8, 4, 128, 128, 128 + 256, 0, 1, None) == 1
+    assert o.prefill_form(1, 8, 4, 128, 2048, 4096, 0, 1, None) == 3
 
 
 def test_which_products_are_taken_in_slices():
