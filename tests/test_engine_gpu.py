@@ -87,15 +87,29 @@ def test_graph_replays_equal_eager_steps(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding_and_first_tokens(tmp_path, dtype):
+@pytest.mark.parametrize("split_from", [None, 4], ids=["", "keys split early"])
+def test_long_decoding_and_first_tokens(tmp_path, dtype, split_from):
     """A short prompt, then hundreds of tokens one by one (several pages, several
     context buckets of the decode graphs); the very first positions of a sequence
-    (position 0 sees itself only) are checked on their own."""
+    (position 0 sees itself only) are checked on their own.  Once more with the keys of a
+    decode step split between workgroups from 128 keys on (contexts this short are not split
+    otherwise), so that the split count changes several times along the way."""
     d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
     cfg, w = plain.read_model_dir(d)
     tokens = random_tokens(600, cfg["vocab_size"], 77)
     want = plain.model_logits_fast(tokens, w, cfg)
     runner = make_runner(d, dtype, 16, 40)
+    if split_from:
+        runner.model.ctx.ops.DECODE_MIN_STEPS_TO_SPLIT = split_from
+        runner.model.ctx.ops.DECODE_MIN_STEPS_PER_SPLIT = 2
+    try:
+        _long_decoding(runner, tokens, want, dtype)
+    finally:
+        for name in ("DECODE_MIN_STEPS_TO_SPLIT", "DECODE_MIN_STEPS_PER_SPLIT"):
+            runner.model.ctx.ops.__dict__.pop(name, None)
+
+
+def _long_decoding(runner, tokens, want, dtype):
     slot = runner.admit()
     first = runner.step([StepEntry(slot, tokens[:1], [0])]).cpu()
     assert (first.double() - want[:1]).abs().max() < TOL[dtype]
