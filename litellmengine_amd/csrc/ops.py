@@ -223,8 +223,7 @@ class HipOps:
                 slices = self.slices_for(M, N, K)
                 if slices:
                     return self.linear_slices(x, weight, slices)
-            skinny = K % 8 == 0 and not self.force_library_gemm and (
-                M <= self.SKINNY_MAX_ROWS or (M <= 16 and N * K <= self.SKINNY_SMALL_WEIGHT))
+            skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.SKINNY_MAX_ROWS
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
                 self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
