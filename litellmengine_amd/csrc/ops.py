@@ -541,11 +541,12 @@ class HipOps:
     def f32_attention_splits(self, num_seqs: int, num_kv_heads: int, row_blocks: int, max_q_len: int,
                              max_kv_len: int, window: int) -> int:
         """Key splits of the float32 matrix-core kernel: enough workgroups for one round of the CUs
-        (measured: more cost 10 % at batch 8 and at 512-token portions), at least 16 of its 16-key
-        steps each."""
+        (measured: more cost 10 % at batch 8 and at 512-token portions), at least 4 of its 16-key
+        steps each (measured at 512 keys: batch 1 in 2 / 8 splits 20 / 12 us, batch 8 in 2 / 4 splits
+        22 / 18 us)."""
         span = min(max_kv_len, window + max_q_len) if window else max_kv_len
         steps = (span + 15) // 16
-        by_work = max(1, steps // 16)
+        by_work = max(1, steps // 4)
         by_fill = max(1, self.compute_units() // max(1, num_seqs * num_kv_heads * row_blocks))
         return int(min(by_work, by_fill, 64))
 
