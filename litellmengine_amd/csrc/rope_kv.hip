@@ -231,25 +231,25 @@ __global__ __launch_bounds__(256) void v_write_transposed_kernel(const bf16_t* _
                              blockIdx.y, tile, s_slot);
 }
 
-// The same for a rotation over the whole head (rot == d): a lane holds four elements of the
-// low half and their four partners of the high half, so the rotation needs no exchange between
-// lanes, and one (cos, sin) pair serves both partners.
-typedef bf16_t rbf16x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void load_weights4(const void* w, int e, int dtype, float (&out)[4]) {
+// The same for a rotation over the whole head (rot == d): a lane holds eight elements of the
+// low half and their eight partners of the high half (16-byte loads and stores), so the rotation
+// needs no exchange between lanes, and one (cos, sin) pair serves both partners.  `per_token`
+// heads of a token are this kernel's: q and k, and v too unless the transposing workgroups take it.
+__device__ __forceinline__ void load_weights8(const void* w, int e, int dtype, float (&out)[8]) {
     if (dtype == LLE_F32) {
-        const float4 v = *(const float4*)((const float*)w + e);
-        out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+        const float4 a = *(const float4*)((const float*)w + e), b = *(const float4*)((const float*)w + e + 4);
+        out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w, out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
     } else {
-        const rbf16x4 v = *(const rbf16x4*)((const bf16_t*)w + e);
+        const rbf16x8 v = *(const rbf16x8*)((const bf16_t*)w + e);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = (float)v[i];
+        for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
     }
 }
 __global__ __launch_bounds__(256) void qk_norm_rope_write_pair_kernel(
     const bf16_t* __restrict__ qkv, const int32_t* __restrict__ slots, const void* __restrict__ q_weight,
     const void* __restrict__ k_weight, int weight_dtype, const float* __restrict__ cos_sin, float eps,
     bf16_t* __restrict__ q_out, bf16_t* __restrict__ kv_layer, int nq, int nkv, int d, int page_size,
-    int64_t page_stride, int write_kv, int total_heads, int head_blocks, int N) {
+    int64_t page_stride, int write_kv, int64_t total_heads, int per_token, int head_blocks, int N) {
     // write_kv == 2: the workgroups after the first `head_blocks` take the V heads of 16 tokens and
     // one kv head each into the transposed pages (the same launch: the two kinds of work overlap)
     if ((int)blockIdx.x >= head_blocks) {
@@ -260,60 +260,61 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_pair_kernel(
                                  vb % nkv, tile, s_slot);
         return;
     }
-    const int lph = d / 8;  // lanes per head
+    const int lph = d / 16;  // lanes per head
     const int lane = threadIdx.x % LLE_WAVE;
     const int heads_per_wave = LLE_WAVE / lph;
     const int64_t gw = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LLE_WAVE;
     const int64_t flat = gw * heads_per_wave + lane / lph;  // (token, head)
     const int hl = lane % lph;
-    const int per_token = nq + 2 * nkv;
-    const bool live = flat < (int64_t)total_heads;
+    const bool live = flat < total_heads;
     const int64_t n = live ? flat / per_token : 0;
     const int head = live ? (int)(flat - n * per_token) : 0;
     const bool is_q = head < nq;
     const bool is_k = !is_q && head < nq + nkv;
     const int half = d / 2;
-    const int e_lo = 4 * hl, e_hi = half + 4 * hl;
+    const int e_lo = 8 * hl, e_hi = half + 8 * hl;
 
-    float lo[4], hi[4];
+    float lo[8], hi[8];
     {
-        const bf16_t* src = qkv + (n * per_token + head) * d;
-        const rbf16x4 a = *(const rbf16x4*)(src + e_lo), b = *(const rbf16x4*)(src + e_hi);
+        const bf16_t* src = qkv + (n * (nq + 2 * nkv) + head) * d;
+        const rbf16x8 a = *(const rbf16x8*)(src + e_lo), b = *(const rbf16x8*)(src + e_hi);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) lo[i] = (float)a[i], hi[i] = (float)b[i];
+        for (int i = 0; i < 8; ++i) lo[i] = (float)a[i], hi[i] = (float)b[i];
     }
     if (is_q || is_k) {
+        // the rotation table is asked for beside the row itself
+        const float4* tab = (const float4*)(cos_sin + (n * half + e_lo) * 2);  // (cos, sin) of e_lo .. e_lo + 7
+        const float4 t0 = tab[0], t1 = tab[1], t2 = tab[2], t3 = tab[3];
         const void* w = is_q ? q_weight : k_weight;
         if (w) {
             float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ss += lo[i] * lo[i] + hi[i] * hi[i];
+            for (int i = 0; i < 8; ++i) ss += lo[i] * lo[i] + hi[i] * hi[i];
             for (int o = 1; o < lph; o <<= 1) ss += __shfl_xor(ss, o, LLE_WAVE);
             const float inv = 1.0f / sqrtf(ss / (float)d + eps);
-            float wl[4], wh[4];
-            load_weights4(w, e_lo, weight_dtype, wl);
-            load_weights4(w, e_hi, weight_dtype, wh);
+            float wl[8], wh[8];
+            load_weights8(w, e_lo, weight_dtype, wl);
+            load_weights8(w, e_hi, weight_dtype, wh);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) lo[i] = lo[i] * inv * wl[i], hi[i] = hi[i] * inv * wh[i];
+            for (int i = 0; i < 8; ++i) lo[i] = lo[i] * inv * wl[i], hi[i] = hi[i] * inv * wh[i];
         }
-        const float4* tab = (const float4*)(cos_sin + (n * half + e_lo) * 2);  // (cos, sin) of e_lo .. e_lo + 3
-        const float4 t0 = tab[0], t1 = tab[1];
-        const float cs[4] = {t0.x, t0.z, t1.x, t1.z}, sn[4] = {t0.y, t0.w, t1.y, t1.w};
+        const float cs[8] = {t0.x, t0.z, t1.x, t1.z, t2.x, t2.z, t3.x, t3.z};
+        const float sn[8] = {t0.y, t0.w, t1.y, t1.w, t2.y, t2.w, t3.y, t3.w};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
             const float a = lo[i], b = hi[i];
             lo[i] = a * cs[i] - b * sn[i];
             hi[i] = b * cs[i] + a * sn[i];
         }
     }
     if (!live) return;
-    rbf16x4 ylo, yhi;
+    rbf16x8 ylo, yhi;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ylo[i] = (bf16_t)lo[i], yhi[i] = (bf16_t)hi[i];
+    for (int i = 0; i < 8; ++i) ylo[i] = (bf16_t)lo[i], yhi[i] = (bf16_t)hi[i];
     if (is_q) {
         bf16_t* dst = q_out + (n * nq + head) * d;
-        *(rbf16x4*)(dst + e_lo) = ylo;
-        *(rbf16x4*)(dst + e_hi) = yhi;
+        *(rbf16x8*)(dst + e_lo) = ylo;
+        *(rbf16x8*)(dst + e_hi) = yhi;
         return;
     }
     if (!write_kv) return;
@@ -324,12 +325,12 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_pair_kernel(
     bf16_t* page_base = kv_layer + page * page_stride;
     if (is_k) {
         bf16_t* dst = page_base + ((int64_t)(head - nq) * page_size + off) * d;
-        *(rbf16x4*)(dst + e_lo) = ylo;
-        *(rbf16x4*)(dst + e_hi) = yhi;
+        *(rbf16x8*)(dst + e_lo) = ylo;
+        *(rbf16x8*)(dst + e_hi) = yhi;
     } else if (write_kv == 1) {
         bf16_t* v = page_base + ((int64_t)nkv + (head - nq - nkv)) * page_size * d + off;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 8; ++i) {
             v[(int64_t)(e_lo + i) * page_size] = ylo[i];
             v[(int64_t)(e_hi + i) * page_size] = yhi[i];
         }
@@ -372,20 +373,22 @@ extern "C" int lle_qk_norm_rope_write(const void* qkv, const void* slots,
         // many tokens: V goes through the transposing kernel (16-byte stores into the pages)
         const bool split_v = write_kv && N >= 64 && page_size % 8 == 0 && (N + VW_TOKENS - 1) / VW_TOKENS <= 0x7fffffff;
         const int64_t v_blocks = split_v ? (int64_t)((N + VW_TOKENS - 1) / VW_TOKENS) * nkv : 0;
-        if (rot == d && blocks + v_blocks <= 0x7fffffff) {
-            qk_norm_rope_write_pair_kernel<<<(unsigned)(blocks + v_blocks), 256,
-                                             split_v ? VW_TOKENS * (d + 2) * sizeof(bf16_t) : 0, stream>>>(
+        if (rot == d) {
+            // the pair kernel: 16 elements a lane; with the transposing workgroups in the same launch
+            // the V heads are theirs alone (without a cache write nobody needs them)
+            const bool own_v = write_kv && !split_v;
+            const int per_token = nq + nkv + (own_v ? nkv : 0);
+            const int64_t pair_heads = (int64_t)N * per_token;
+            const int pair_heads_per_block = 4 * (LLE_WAVE / (d / 16));
+            const int64_t pair_blocks = (pair_heads + pair_heads_per_block - 1) / pair_heads_per_block;
+            const bool one_launch = pair_blocks + v_blocks <= 0x7fffffff;
+            qk_norm_rope_write_pair_kernel<<<(unsigned)(one_launch ? pair_blocks + v_blocks : pair_blocks), 256,
+                                             split_v && one_launch ? VW_TOKENS * (d + 2) * sizeof(bf16_t) : 0, stream>>>(
                 (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, eps,
                 (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
-                write_kv ? (split_v ? 2 : 1) : 0, total_heads, blocks, N);
-            LLE_RETURN_LAUNCH_STATUS();
-        }
-        if (rot == d)
-            qk_norm_rope_write_pair_kernel<<<blocks, 256, 0, stream>>>(
-                (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, eps,
-                (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
-                write_kv ? (split_v ? 2 : 1) : 0, total_heads, blocks, N);
-        else
+                write_kv ? (split_v ? 2 : 1) : 0, pair_heads, per_token, (int)pair_blocks, N);
+            if (one_launch) LLE_RETURN_LAUNCH_STATUS();
+        } else
             qk_norm_rope_write_vec_kernel<<<blocks, 256, 0, stream>>>(
                 (const bf16_t*)qkv, (const int32_t*)slots, q_weight, k_weight, weight_dtype, (const float*)cos_sin, rot,
                 eps, (bf16_t*)q_out, (bf16_t*)kv_layer, nq, nkv, d, page_size, page_stride,
