@@ -63,7 +63,7 @@ __device__ __forceinline__ float4 load_weight4(const void* w, int i, int dtype) 
 #define NORM_CHUNKS 8
 // `delta` may come as `slices` partial sums of type TD, `slice_stride` elements apart (a product
 // over slices of K leaves them so): they are added in slice order.
-template <typename T, typename TD = T>
+template <typename T, typename TD = T, bool SLICED = false>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ hidden, const TD* __restrict__ delta,
                                                               const int32_t* __restrict__ rows,
                                                               const void* __restrict__ weight, int weight_dtype,
@@ -81,28 +81,72 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         const int i = (k * 256 + threadIdx.x) * 4;
         if (i < H) wv[k] = load_weight4(weight, i, weight_dtype);
     }
-#pragma unroll
-    for (int k = 0; k < NORM_CHUNKS; ++k) {
-        const int i = (k * 256 + threadIdx.x) * 4;
-        if (i < H) {
-            float4 x = *(const float4*)(h + i);
-            if (dl) {
-                float4 d = Quad<TD>::load(dl + i);
-                for (int sl = 1; sl < slices; ++sl) {
-                    const float4 e = Quad<TD>::load(dl + sl * slice_stride + i);
-                    d.x += e.x;
-                    d.y += e.y;
-                    d.z += e.z;
-                    d.w += e.w;
-                }
-                x.x += d.x;
-                x.y += d.y;
-                x.z += d.z;
-                x.w += d.w;
-                if (!rows) *(float4*)(h + i) = x;
+    if constexpr (SLICED) {
+        // all of a row's loads of one kind are asked for together (a load that waits for the one before
+        // it pays the memory's latency once more): the row and the first slice, then slice by slice
+        float4 d[NORM_CHUNKS];
+    #pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                v[k] = *(const float4*)(h + i);
+                if (dl) d[k] = Quad<TD>::load(dl + i);
             }
-            v[k] = x;
-            ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        }
+        if (dl) {
+    #pragma unroll 2
+            for (int sl = 1; sl < slices; ++sl) {
+                float4 e[NORM_CHUNKS];
+    #pragma unroll
+                for (int k = 0; k < NORM_CHUNKS; ++k) {
+                    const int i = (k * 256 + threadIdx.x) * 4;
+                    if (i < H) e[k] = Quad<TD>::load(dl + sl * slice_stride + i);
+                }
+    #pragma unroll
+                for (int k = 0; k < NORM_CHUNKS; ++k) {
+                    const int i = (k * 256 + threadIdx.x) * 4;
+                    if (i < H) {
+                        d[k].x += e[k].x;
+                        d[k].y += e[k].y;
+                        d[k].z += e[k].z;
+                        d[k].w += e[k].w;
+                    }
+                }
+            }
+        }
+    #pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                float4 x = v[k];
+                if (dl) {
+                    x.x += d[k].x;
+                    x.y += d[k].y;
+                    x.z += d[k].z;
+                    x.w += d[k].w;
+                    if (!rows) *(float4*)(h + i) = x;
+                }
+                v[k] = x;
+                ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                float4 x = *(const float4*)(h + i);
+                if (dl) {
+                    const float4 d = Quad<TD>::load(dl + i);
+                    x.x += d.x;
+                    x.y += d.y;
+                    x.z += d.z;
+                    x.w += d.w;
+                    if (!rows) *(float4*)(h + i) = x;
+                }
+                v[k] = x;
+                ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+            }
         }
     }
     ss = block_sum(ss, red);
@@ -127,11 +171,11 @@ extern "C" int lle_add_rmsnorm_sums(void* hidden, const void* sums, int slices, 
     if (R <= 0) return 0;
     if (H % 4 != 0 || H > 256 * 4 * NORM_CHUNKS || slices < 1 || !sums) return (int)hipErrorInvalidValue;
     if (dtype == LLE_F32)
-        add_rmsnorm_vec_kernel<float, float><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
+        add_rmsnorm_vec_kernel<float, float, true><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
                                                                      (const int32_t*)rows, weight, weight_dtype,
                                                                      (float*)out, H, eps, slices, slice_stride);
     else
-        add_rmsnorm_vec_kernel<bf16_t, float><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
+        add_rmsnorm_vec_kernel<bf16_t, float, true><<<R, 256, 0, stream>>>((float*)hidden, (const float*)sums,
                                                                       (const int32_t*)rows, weight, weight_dtype,
                                                                       (bf16_t*)out, H, eps, slices, slice_stride);
     LLE_RETURN_LAUNCH_STATUS();

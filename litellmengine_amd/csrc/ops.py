@@ -252,22 +252,37 @@ class HipOps:
 
     def slices_for(self, M: int, N: int, K: int) -> int:
         """In how many slices of K the product of 17 to 128 rows with a weight [N, K] is taken
-        (see linear_slices), or 0 where the library product stays: the workgroups, N / 64 x slices,
-        have to fill the CUs in whole rounds (at least 0.85 of them), which weights with few rows
-        per CU do (o_proj, down_proj) and wide ones need no slices for."""
+        (see linear_slices), or 0 where the library product stays.  Weights with rows enough for
+        every CU need no slices.  For the others the slice count is the one that a small model of
+        the kernel's time likes best (rounds of N / 64 x slices workgroups over the CUs, each
+        taking in its W and X at what a CU takes in, plus the way of the partial sums to the norm
+        and back), and it is used where the workgroups fill the CUs in whole rounds (at least
+        0.85 of them: o_proj, down_proj of the 8B sizes), or where K is at least twice N and the
+        weight is not small: there the library's tiles are too few for the CUs and it does not
+        split K (measured at 64 rows: down_proj of the 32B sizes, 5120 x 25600, in 5 slices 76 us
+        against the library's 158; of the 14B sizes, 5120 x 17408, in 17 slices 70 against 132)."""
         if not (self.SLICED_MIN_ROWS <= M <= self.SLICED_MAX_ROWS) or N % 64 != 0 or self.force_library_gemm:
             return 0
         units = self.compute_units()
-        if N // 64 > units // 2:  # enough rows for the library's own tiles
+        groups = N // 64
+        if groups > units // 2 or K % self.SLICED_UNIT != 0:  # (rows enough for the library's own tiles)
             return 0
-        for slices in (2, 3, 4, 6, 8):
-            if K % (self.SLICED_UNIT * slices) != 0:
+        parts = K // self.SLICED_UNIT
+        rows = 32 if M <= 32 else 64 if M <= 64 else 96 if M <= 96 else 128  # the kernel's tiles of X
+        best, best_time, best_fill = 0, 0.0, 0.0
+        for slices in range(1, min(parts, 32) + 1):
+            if parts % slices != 0:
                 continue
-            groups = (N // 64) * slices
-            rounds = -(-groups // units)
-            if groups >= 0.85 * rounds * units:
-                return slices
+            rounds = -(-groups * slices // units)
+            taken_in = (64 + rows) * (K // slices) * 2  # bytes of W and X through a CU, at about 29 GB/s
+            seconds = rounds * (3e-6 + taken_in / 29e9) + slices * M * N * 8 / 5e12
+            if best == 0 or seconds < best_time:
+                best, best_time, best_fill = slices, seconds, groups * slices / (rounds * units)
+        if best_fill >= 0.85 or (K >= 2 * N and N * K >= self.SLICED_LONG_K_MIN_WEIGHT):
+            return best
         return 0
+
+    SLICED_LONG_K_MIN_WEIGHT = 1 << 23  # elements: below, a launch is as short as a launch can be either way
 
     def linear_slices(self, x, weight, slices: int) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T as float32 partial sums over `slices` equal parts of K:

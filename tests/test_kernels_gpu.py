@@ -150,7 +150,7 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
 
 
 @pytest.mark.parametrize("M", [17, 31, 32, 33, 48, 64, 65, 81, 96, 97, 128])
-@pytest.mark.parametrize("N,K,slices", [(4096, 4096, 4), (4096, 12288, 4), (320, 2048, 2), (64, 1024, 1), (128, 3072, 3)])
+@pytest.mark.parametrize("N,K,slices", [(4096, 4096, 4), (4096, 12288, 4), (320, 2048, 2), (64, 1024, 1), (128, 3072, 3), (640, 17408, 17)])
 def test_product_in_slices_of_k(M, N, K, slices):
     """The product of 17 to 128 rows taken in slices of K: the float32 partial sums add up to the
     float64 product, each slice is the product over its own columns, and the residual add + norm
@@ -218,6 +218,11 @@ def test_which_products_are_taken_in_slices():
     assert o.slices_for(64, 64 * units, 4096) == 0      # wide: rows enough for every CU
     assert o.slices_for(64, n + 8, 4096) == 0           # no multiple of 64 rows
     assert o.slices_for(64, n, 4096 + 256) == 0         # no whole slices
+    if units == 256:
+        # a long K beside few rows (down_proj of the 32B and 14B sizes): slices although the workgroups fill
+        # no whole rounds; a square weight in a round and a quarter (o_proj of the 32B sizes) stays the library's
+        assert o.slices_for(64, 5120, 25600) == 5 and o.slices_for(64, 5120, 17408) == 17
+        assert o.slices_for(64, 5120, 8192) == 0 and o.slices_for(64, 1024, 3072) == 0
     x = rnd((40, 4096), torch.bfloat16, 65)
     w = rnd((n, 4096), torch.bfloat16, 66, 0.05)
     assert o.linear(x, w).shape == (40, n)                       # a caller that said nothing gets the product
