@@ -15,17 +15,22 @@ def cpu_engine(d, **kw):
     return LLMEngine(model, **kw)
 
 
-def test_greedy_generation_equals_full_recompute(tmp_path):
-    """Workload of the tiny configuration A: prompts 5/9/17, 8 greedy steps, page size 4."""
-    d = make_model_dir(tmp_path, "A")
+@pytest.mark.parametrize("which,page_size", [("A", 4), ("C", 16)])
+def test_greedy_generation_equals_full_recompute(tmp_path, which, page_size):
+    """Workload of the tiny configuration A: prompts 5/9/17, 8 greedy steps, page size 4.  (With
+    tied embeddings and random weights A mostly repeats a prompt's last token; C, with an output
+    head of its own, goes through different tokens.)"""
+    d = make_model_dir(tmp_path, which)
     cfg, w = plain.read_model_dir(d)
     prompts = [random_tokens(n, 256, i) for i, n in enumerate((5, 9, 17))]
     want = [plain.generate_greedy(p, w, cfg, 8) for p in prompts]
-    eng = cpu_engine(d, page_size=4, num_pages=24, max_requests=3)
+    if which == "C":
+        assert len(set(sum(want, []))) >= 6
+    eng = cpu_engine(d, page_size=page_size, num_pages=24, max_requests=3)
     assert eng.generate(prompts, 8) == want
     # each alone == among the others (tests/test_paged_generate_engine.cpp:428-552)
     for p, x in zip(prompts, want):
-        assert cpu_engine(d, page_size=4, num_pages=24, max_requests=1).generate([p], 8) == [x]
+        assert cpu_engine(d, page_size=page_size, num_pages=24, max_requests=1).generate([p], 8) == [x]
 
 
 def test_chunked_prefill_and_preemption_do_not_change_tokens(tmp_path):
@@ -103,13 +108,14 @@ def test_parked_sessions_lose_their_cache_before_running_requests_are_preempted(
 
 
 def test_eos_is_appended_and_ends_the_request(tmp_path):
-    d = make_model_dir(tmp_path, "A")
+    d = make_model_dir(tmp_path, "C")
     cfg, w = plain.read_model_dir(d)
     p = random_tokens(6, 256, 3)
     free = plain.generate_greedy(p, w, cfg, 8)
-    eos = free[2]
-    cut = free[: free.index(eos) + 1]
-    assert cpu_engine(d, page_size=4, num_pages=8, max_requests=1).generate([p], 8, eos_token_id=eos) == [cut]
+    at = next(i for i in range(2, 8) if free[i] not in free[:i])  # a token that is new where it stands
+    eos = free[at]
+    cut = free[: at + 1]
+    assert cpu_engine(d, page_size=16, num_pages=8, max_requests=1).generate([p], 8, eos_token_id=eos) == [cut]
 
 
 def test_temperature_draws_do_not_depend_on_the_batch(tmp_path):
