@@ -142,12 +142,14 @@ class ModelRunner:
     def _capture(self, layout: StepLayout, host: torch.Tensor, bucket: int) -> _DecodeGraph:
         buf = host.to(self.device)
         state = state_on(buf, layout, self.cache, max_kv_len=bucket, with_seqs=False)
-        # run the step for real first (twice: library workspaces and lazy kernel set-up happen here);
-        # a decode step is idempotent: it writes the same K/V and yields the same logits
+        # run the step for real first (the library picks its products for these sizes and takes its
+        # workspaces here, kernels set themselves up: none of that may happen under capture; the very
+        # first capture runs it twice); a decode step is idempotent: it writes the same K/V and yields
+        # the same logits
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(side):
-            for _ in range(2):
+            for _ in range(2 if self.num_captures == 0 else 1):
                 self.model.forward(state, self.cache)
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
