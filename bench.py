@@ -7,6 +7,7 @@
     python bench.py --sizes 32b | --sizes 0p6b                    # the decode workload at other layer sizes
     python bench.py --workload reference-0p6b [--dtype float32]   # the reference's own benchmark shape
     python bench.py --workload mixed-32b [--layers L]             # a prompt chunk beside 63 decoded tokens
+    python bench.py --workload serving                            # requests of many lengths arriving over time
 
 A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
@@ -278,6 +279,71 @@ def mixed_workload(args):
     return 0
 
 
+def serving_workload(args):
+    """Requests of many lengths arriving over time, through the engine's own scheduler, at the
+    Qwen3-8B layer sizes: 200 requests, prompts of 30 to 3050 tokens, 16 to 256 new tokens each,
+    one arriving every second step, at most 64 live, a budget of 2048 tokens a step.  The whole run
+    is timed (prompt portions beside decoded tokens, graph captures included); all tokens / time."""
+    import collections
+    import random
+
+    import torch
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.engine import LLMEngine
+    from litellmengine_amd.models import random_model
+
+    cfg = Qwen3Config.from_dict(dict(SIZES, num_hidden_layers=args.layers))
+    model = random_model(cfg, seed=0, dtype=args.dtype)
+    rng = random.Random(5)
+    requests, live, every = 200, 64, 2
+    sizes = [(rng.choice([30, 100, 300, 700, 1500, 3000]) + rng.randint(0, 50), rng.choice([16, 64, 128, 256]))
+             for _ in range(requests)]
+    longest = max(p + g for p, g in sizes)
+    pages_each = (longest + PAGE_SIZE - 1) // PAGE_SIZE + 1
+    engine = LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_each * live, max_requests=live,
+                       max_tokens_per_step=PREFILL_TOKENS, max_pages_per_request=pages_each)
+    todo = [(random_prompts(1, p, cfg.vocab_size, 100 + i)[0], g) for i, (p, g) in enumerate(sizes)]
+    kinds = collections.defaultdict(lambda: [0, 0.0])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = 0
+    while todo or engine.has_work():
+        if todo and steps % every == 0:
+            prompt, new = todo.pop(0)
+            engine.add_request(prompt, new)
+        before = sum(r.cached_len for r in engine.scheduler.requests.values())
+        captures = engine.runner.num_captures
+        ts = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - ts
+        ran = sum(r.cached_len for r in engine.scheduler.requests.values()) - before
+        kind = ("capture" if engine.runner.num_captures > captures else
+                "le64" if ran <= 64 else "le256" if ran <= 256 else "le1024" if ran <= 1024 else "gt1024")
+        kinds[kind][0] += 1
+        kinds[kind][1] += dt
+        steps += 1
+    total = time.perf_counter() - t0
+    new_tokens = sum(g for _, g in sizes)
+    all_tokens = sum(p + g for p, g in sizes)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": "tokens/s, prompts included, of 200 requests (prompts of 30-3050 tokens, 16-256 new tokens) "
+                  "arriving one every second step, at most 64 live, Qwen3-8B sizes",
+        "value": round(all_tokens / total, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 0,
+        "ms_per_step": round(total / steps * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": short, "data": "synthetic: seeded random weights, uniform random token ids, seeded lengths",
+        "config": flat_config(cfg, SIZES["num_hidden_layers"], model="Qwen3-8B sizes (random weights)",
+                              global_batch=live, requests=requests, token_budget=PREFILL_TOKENS),
+        "new_tokens_per_s": round(new_tokens / total, 1), "seconds": round(total, 3),
+        "graph_captures": engine.runner.num_captures,
+        "steps_by_tokens": {k: {"steps": n, "ms_each": round(t / n * 1e3, 2), "share": round(t / total, 3)}
+                            for k, (n, t) in sorted(kinds.items())},
+    }))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -290,7 +356,7 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b"],
                     help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B")
-    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving"],
                     help="decode (default: the headline line), the reference's own benchmark shape at Qwen3-0.6B "
                          "sizes, or a mixed prompt-portion + decode step at Qwen3-32B sizes")
     args = ap.parse_args()
@@ -304,6 +370,8 @@ def main():
         if args.workload == "reference-0p6b":
             args.steps, args.warmup = min(args.steps, 5), min(args.warmup, 1)
             return reference_workload(args)
+        if args.workload == "serving":
+            return serving_workload(args)
         args.steps, args.warmup = min(args.steps, 3), min(args.warmup, 1)
         return mixed_workload(args)
 
