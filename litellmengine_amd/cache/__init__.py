@@ -1,4 +1,4 @@
-from .manager import CacheGroup, CacheManager, LayerCache
+from .manager import CacheGroup, CacheManager, GroupSizes, LayerCache
 from .page_pool import OutOfPages, PagePool
 
-__all__ = ["CacheGroup", "CacheManager", "LayerCache", "OutOfPages", "PagePool"]
+__all__ = ["CacheGroup", "CacheManager", "GroupSizes", "LayerCache", "OutOfPages", "PagePool"]

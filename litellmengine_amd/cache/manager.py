@@ -169,11 +169,30 @@ class LayerCache:
         raise KeyError(f"the cache record has no field {name!r}")
 
 
+@dataclasses.dataclass(frozen=True)
+class GroupSizes:
+    """Page size and pool of one cache group, where the caller wants to set them."""
+
+    page_size: Optional[int] = None
+    num_pages: Optional[int] = None
+
+
 class CacheManager:
     def __init__(self, model, *, page_size: int, num_pages: int, max_requests: int,
-                 max_pages_per_request: Optional[int] = None, dtype: torch.dtype, device):
-        """`model` is a models.decoder.DecoderLM (its plan and mixers say what is
-        needed); every group gets `num_pages` pages of `page_size` tokens."""
+                 max_pages_per_request: Optional[int] = None, dtype: torch.dtype, device,
+                 max_tokens_per_step: Optional[int] = None,
+                 group_sizes: Optional[Dict[CacheSpec, GroupSizes]] = None):
+        """`model` is a models.decoder.DecoderLM (its plan and mixers say what is needed).
+        `page_size` and `num_pages` give the page size and the capacity (num_pages * page_size
+        tokens) of a group that asks for nothing else; every group has a page size and a pool
+        of its own:
+          * page size: `group_sizes[spec].page_size`, else the spec's own, else `page_size`;
+          * pool: `group_sizes[spec].num_pages`, else pages for the same number of tokens; a
+            group with a window needs no more than the window and one step's tokens per
+            request, and is sized so when `max_tokens_per_step` says how long a step may be
+            (the reference has one geometry and one pool for all layers,
+            src/engine/paged_kv_cache.cpp:26-52).
+        `max_pages_per_request` counts pages of `page_size` tokens: the longest request."""
         if page_size <= 0:
             raise ValueError("--page-size must be positive")  # src/main.cpp:62-64
         device = torch.device(device)
@@ -183,29 +202,41 @@ class CacheManager:
         self.device = device
         self.dtype = dtype
         max_pages_per_request = max_pages_per_request or num_pages
+        capacity, longest = num_pages * page_size, max_pages_per_request * page_size
 
         by_spec: Dict[CacheSpec, List[int]] = {}
         for cache_id, mixer in sorted(model.cache_layers().items()):
             spec = mixer.cache_spec()
             if spec is not None:
                 by_spec.setdefault(spec, []).append(cache_id)
-        self.groups: List[CacheGroup] = [
-            CacheGroup(g, spec, ids, page_size, num_pages, max_requests, max_pages_per_request, dtype, device)
-            for g, (spec, ids) in enumerate(by_spec.items())
-        ]
+        self.groups: List[CacheGroup] = []
+        for g, (spec, ids) in enumerate(by_spec.items()):
+            asked = (group_sizes or {}).get(spec, GroupSizes())
+            P = asked.page_size or spec.page_size or page_size
+            if P <= 0:
+                raise ValueError("a group's page size must be positive")
+            pages = asked.num_pages
+            if pages is None:
+                pages = -(-capacity // P)
+                if spec.window is not None and max_tokens_per_step is not None:
+                    # positions past - window + 1 .. past + step - 1 of a request, wherever they start in a page
+                    each = -(-(spec.window - 1 + max_tokens_per_step) // P) + 1
+                    pages = min(pages, max_requests * each)
+            self.groups.append(CacheGroup(g, spec, ids, P, pages, max_requests, -(-longest // P), dtype, device))
         where: Dict[int, Tuple[CacheGroup, int]] = {}
         for group in self.groups:
             for n, cache_id in enumerate(group.cache_ids):
                 where[cache_id] = (group, n)
 
-        # state rows belong to a cache id too: every entry that names it shares them
+        # state rows belong to a cache id too: every entry that names it shares them; row `pad_slot`
+        # (one more than there are request slots) belongs to nobody: the rows that pad a batch use it
         self.states: Dict[int, torch.Tensor] = {}
         self._layers: List[LayerCache] = []
         for entry in model.plan:
             mixer = model.blocks[entry.block].mixer
             sspec: Optional[StateSpec] = mixer.state_spec()
             if sspec is not None and entry.cache not in self.states:
-                self.states[entry.cache] = torch.zeros((max_requests,) + tuple(sspec.shape), dtype=sspec.dtype, device=device)
+                self.states[entry.cache] = torch.zeros((max_requests + 1,) + tuple(sspec.shape), dtype=sspec.dtype, device=device)
             group, n = where.get(entry.cache, (None, 0))
             self._layers.append(
                 LayerCache(group, None if group is None or group.kv is None else group.kv[n], entry.writes,

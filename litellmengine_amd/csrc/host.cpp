@@ -241,7 +241,8 @@ void lle_pt_take_pending(void* h, int32_t* index, int32_t* pages) {
 int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int32_t* q_len, const int32_t* tokens,
                     int vocab_size, int R, const int32_t* logit_rows, int G, void* const* groups, int pad,
                     int pad_slot, int32_t* out, int64_t* info) {
-    if (S <= 0 || R < 0 || G < 0 || pad < 0 || (pad > 0 && pad_slot < 0)) return LLE_HOST_BAD_ARGUMENT;
+    // (no request at all is allowed when the batch is padding only: the warm-up of a graph's kernels)
+    if (S < 0 || (S == 0 && pad <= 0) || R < 0 || G < 0 || pad < 0 || (pad > 0 && pad_slot < 0)) return LLE_HOST_BAD_ARGUMENT;
     int64_t N = 0;
     for (int s = 0; s < S; ++s) {
         if (q_len[s] <= 0 || past[s] < 0) {

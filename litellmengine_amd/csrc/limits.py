@@ -3,6 +3,9 @@ together (a model that a kernel would refuse at its first step is refused when i
 and `ops.py` checks them again before a launch.  Nothing here touches the GPU."""
 
 MAX_HEAD_DIM = 256  # the attention kernels keep a head's elements in four registers per lane
+# the widest row whose partial sums (a product taken in slices of K) the residual add + norm adds
+# up: 256 threads x 4 elements x NORM_CHUNKS of norm.hip, and a multiple of 4
+MAX_SUMMED_NORM_WIDTH = 8192
 
 
 def check_head_dim(head_dim: int, rotary_dim: int = 0) -> None:

@@ -10,9 +10,9 @@ from typing import Optional
 
 import torch
 
-from ..parts.base import Prenormed
+from ..parts.base import PartialSums, Prenormed
 from . import build
-from .limits import MAX_HEAD_DIM
+from .limits import MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH
 
 F32, BF16 = 0, 1
 _P = ctypes.c_void_p
@@ -109,17 +109,19 @@ class HipOps:
     # -- norms ---------------------------------------------------------------
     def add_rmsnorm(self, hidden, delta, weight, eps: float, out_dtype, rows=None) -> torch.Tensor:
         """hidden float32 [N, H] (+ delta [N, H] of out_dtype, or float32 partial sums
-        [slices, N, H] that are added in slice order) -> norm * weight, out_dtype.
+        [slices, N, H], bare or as PartialSums, that are added in slice order) -> norm * weight, out_dtype.
         Without `rows` the sum is written back to `hidden` and every row is normed;
         with `rows` (int32 [R]) only those rows are read and nothing is written back."""
         _dev(hidden, "hidden", torch.float32)
         _dev(weight, "norm weight")
         N, H = hidden.shape
         _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        if isinstance(delta, PartialSums):
+            delta = delta.sums
         sums = delta is not None and delta.dim() == 3  # partial sums of a product taken in slices of K
         if sums:
             _dev(delta, "partial sums", torch.float32)
-            _need(delta.shape[1:] == hidden.shape and H % 4 == 0 and H <= 8192,
+            _need(delta.shape[1:] == hidden.shape and H % 4 == 0 and H <= MAX_SUMMED_NORM_WIDTH,
                   f"partial sums {list(delta.shape)} do not fit the residual stream {list(hidden.shape)}")
         elif delta is not None:
             _dev(delta, "delta", out_dtype)
@@ -203,7 +205,7 @@ class HipOps:
 
     def linear(self, x, weight, out_dtype=None, fold=None, sums_ok=False):
         """x [M, K] . weight [N, K]^T -> [M, N].  With `sums_ok` the caller takes the result also as
-        float32 partial sums [slices, M, N] (what add_rmsnorm adds into the residual stream).  float32 operands take a true 32-bit
+        PartialSums (float32 [slices, M, N], what add_rmsnorm adds into the residual stream).  float32 operands take a true 32-bit
         product: few rows the weight-streaming kernel, more rows a tiled kernel, both
         with the float32 matrix instruction; the plain-FMA kernel where K is no multiple of 4.  bfloat16 operands: few rows take the
         weight-streaming matrix-core kernel, more rows the library product; both
@@ -222,7 +224,7 @@ class HipOps:
             if sums_ok and out_dtype == torch.bfloat16:
                 slices = self.slices_for(M, N, K)
                 if slices:
-                    return self.linear_slices(x, weight, slices)
+                    return PartialSums(self.linear_slices(x, weight, slices))
             skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.SKINNY_MAX_ROWS
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
@@ -262,6 +264,8 @@ class HipOps:
         split K (measured at 64 rows: down_proj of the 32B sizes, 5120 x 25600, in 5 slices 76 us
         against the library's 158; of the 14B sizes, 5120 x 17408, in 17 slices 70 against 132)."""
         if not (self.SLICED_MIN_ROWS <= M <= self.SLICED_MAX_ROWS) or N % 64 != 0 or self.force_library_gemm:
+            return 0
+        if N > MAX_SUMMED_NORM_WIDTH:  # the only reader of the partial sums (add_rmsnorm) takes no wider rows
             return 0
         units = self.compute_units()
         groups = N // 64

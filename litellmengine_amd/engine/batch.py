@@ -138,7 +138,7 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
         raise IndexError(f"position {info.value} has no page: the cache was not extended for this step")
     if code != 0:
         raise ValueError(f"the step cannot be laid out: {lib.lle_error_string(code).decode()} (at {info.value})")
-    return StepLayout(host, N + pad, S + pad, R, G, seqs, max(p + n for p, n in zip(past, q_len)))
+    return StepLayout(host, N + pad, S + pad, R, G, seqs, max((p + n for p, n in zip(past, q_len)), default=1))
 
 
 def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:

@@ -25,7 +25,8 @@ class LLMEngine:
         ctx = model.ctx
         self.model = model
         self.cache = CacheManager(model, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
-                                  max_pages_per_request=max_pages_per_request, dtype=ctx.dtype, device=ctx.device)
+                                  max_pages_per_request=max_pages_per_request, dtype=ctx.dtype, device=ctx.device,
+                                  max_tokens_per_step=max_tokens_per_step)
         self.runner = ModelRunner(model, self.cache)
         self.scheduler = Scheduler(self.cache, max_tokens_per_step, prefill_chunk)
         self.sampler = Sampler(ctx.ops, ctx.device)

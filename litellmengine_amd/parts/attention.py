@@ -88,9 +88,8 @@ class PagedAttention(Mixer):
         group = cache.group
         if fused is not None:
             cos_sin, rot = fused
-            can_fuse = getattr(ops, "can_fuse_rope_attention", None)  # an ops object without it never fuses
-            if can_fuse is not None and can_fuse(qkv.dtype, self.d, rot, cache.kv.shape[3], self.nq // self.nkv,
-                                                 step.max_q_len, step.max_kv_len, step.seq_slots.shape[0]):
+            if ops.can_fuse_rope_attention(qkv.dtype, self.d, rot, cache.kv.shape[3], self.nq // self.nkv,
+                                           step.max_q_len, step.max_kv_len, step.seq_slots.shape[0]):
                 # a decode step: norm, rotation, cache write and attention in one launch
                 a = ops.qk_norm_rope_attention(
                     qkv, group.slot_mapping, self.q_norm_w, self.k_norm_w, cos_sin, eps, cache.kv, self.nq,

@@ -49,10 +49,13 @@ class CacheSpec:
     """Per-token cache need of a mixer: a record of named fields for every token.  A page
     holds the fields one after the other, each for all of the page's tokens.  With a
     `window` only the last `window` positions stay needed and pages behind it are given back.
-    Mixers with equal specs share a group of pages and block tables."""
+    `page_size`: tokens per page, if the mixer's kernels want a size of their own (None: the
+    engine's).  Mixers with equal specs share a group of pages and block tables; every group
+    has a page size and a pool of its own."""
 
     fields: Tuple[CacheField, ...]
     window: Optional[int] = None
+    page_size: Optional[int] = None
 
     def __post_init__(self):
         names = [f.name for f in self.fields]
@@ -61,6 +64,8 @@ class CacheSpec:
         for f in self.fields:
             if f.num_heads <= 0 or f.width <= 0:
                 raise ValueError(f"cache field {f.name!r} needs positive sizes")
+        if self.page_size is not None and self.page_size <= 0:
+            raise ValueError("a cache record's page size must be positive")
 
     @property
     def elems_per_token(self) -> int:
@@ -77,15 +82,20 @@ class CacheSpec:
         return k.num_heads, k.width
 
 
-def KVCacheSpec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> CacheSpec:
+def KVCacheSpec(num_kv_heads: int, head_dim: int, window: Optional[int] = None,
+                page_size: Optional[int] = None) -> CacheSpec:
     """Keys and values of `num_kv_heads` heads of `head_dim`, in the layout the attention
     kernels read: K as [head][token][d], V transposed as [head][d][token]."""
-    return CacheSpec((CacheField("k", num_kv_heads, head_dim), CacheField("v", num_kv_heads, head_dim, True)), window)
+    return CacheSpec((CacheField("k", num_kv_heads, head_dim), CacheField("v", num_kv_heads, head_dim, True)), window,
+                     page_size)
 
 
 @dataclasses.dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size per-request state of a mixer (zeroed when a request is admitted)."""
+    """Fixed-size per-request state of a mixer (zeroed when a request is admitted).  The state
+    tensor has one row per request slot and one more, which belongs to nobody: rows that pad a
+    decode batch to a graph's size name it in `step.seq_slots`, and what they leave there is
+    never read by a request."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
@@ -124,13 +134,26 @@ class Prenormed:
     eps: float
 
 
+@dataclasses.dataclass
+class PartialSums:
+    """A product that was taken in slices of its inner dimension and not added up yet:
+    `sums` is float32 [slices, N, width], and the product is their sum in slice order.  Only a
+    Linear made with `to_residual` returns one, and only Norm.forward takes it (it is no tensor:
+    a block that adds its delta by hand fails loudly instead of broadcasting over the slices)."""
+
+    sums: torch.Tensor
+
+    def total(self) -> torch.Tensor:
+        """The product itself, float32 [N, width] (the plain way to take it)."""
+        return self.sums.sum(0)
+
+
 class Norm(Part):
     """forward(hidden, delta) adds `delta` (or nothing) into the 32-bit residual
     stream `hidden` in place and returns the normed rows in the activation type;
     with `rows` only those rows are read and `hidden` is left alone.  `delta` is
-    [N, hidden] in the activation type, or float32 partial sums [slices, N, hidden]
-    that are to be added in slice order (a Linear made with `to_residual` may leave
-    them so; `delta.sum(0)` is the plain way to take them).
+    [N, hidden] in the activation type, or the PartialSums that a Linear made with
+    `to_residual` may leave (`delta.total()` is the plain way to take them).
 
     fold(hidden) may return a NormFold when the step is small enough that the
     products on both sides of the norm can do its work (None: call forward)."""
@@ -166,7 +189,9 @@ class Mixer(Part):
 
     # True if forward() uses only device arrays of the step (no host-side view of
     # the batch, no sizes that depend on the step's values): decode steps of such
-    # mixers may be captured into a graph and replayed.
+    # mixers may be captured into a graph and replayed.  A replay runs forward() once
+    # per step, like a step without graphs: state may be kept and advanced.  What runs
+    # before a capture to warm the kernels up runs on padding rows only.
     graph_safe = False
     # True if forward() takes a Prenormed for x (passing it to one product only) and
     # a keyword `fold` (a NormFold for its last product, whose Prenormed it then returns).

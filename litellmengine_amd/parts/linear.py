@@ -16,8 +16,8 @@ class Linear(Part):
     def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int], optional: bool = False,
                  to_residual: bool = False):
         """`to_residual`: the result is a delta of the residual stream and goes nowhere but into
-        Norm.forward(hidden, delta); it may then come as float32 partial sums [slices, N, out]
-        (a product taken in slices of `in`), which that call adds up."""
+        Norm.forward(hidden, delta); it may then come as parts.base.PartialSums (a product taken
+        in slices of `in`), which that call adds up."""
         self.names = list(names)
         self.in_features = in_features
         self.out_features = list(out_features)
@@ -45,7 +45,7 @@ class Linear(Part):
         """`x` may be a parts.base.Prenormed; with `fold` (a parts.base.NormFold) the result
         is added into the residual stream and comes back as the Prenormed of that norm."""
         if fold is None:
-            if self.to_residual and out_dtype is None and hasattr(self.ctx.ops, "slices_for"):
+            if self.to_residual and out_dtype is None:
                 return self.ctx.ops.linear(x, self.weight, out_dtype, sums_ok=True)
             return self.ctx.ops.linear(x, self.weight, out_dtype)
         return self.ctx.ops.linear(x, self.weight, out_dtype, fold=fold)

@@ -29,7 +29,6 @@ class RMSNorm(Norm):
         return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)
 
     def fold(self, hidden) -> Optional[NormFold]:
-        can = getattr(self.ctx.ops, "can_fold_norm", None)  # an ops object without it never folds
-        if can is None or not can(hidden.shape[0], self.size, self.ctx.dtype):
+        if not self.ctx.ops.can_fold_norm(hidden.shape[0], self.size, self.ctx.dtype):
             return None
         return NormFold(hidden, self.weight, self.eps)

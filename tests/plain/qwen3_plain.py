@@ -336,7 +336,9 @@ def first_layer_attention_probs(ids, w, cfg) -> torch.Tensor:
     return torch.softmax(scores.masked_fill(~allowed[None], float("-inf")), dim=-1)
 
 
-def model_logits_fast(ids, w, cfg, positions=None) -> torch.Tensor:
+def model_logits_fast(ids, w, cfg, positions=None, rows=None) -> torch.Tensor:
+    """`rows`: only these positions go through the final norm and the head (long sequences,
+    wide vocabularies); the result then has one row for each of them, in their order."""
     T = len(ids)
     positions = list(range(T)) if positions is None else positions
     nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -357,6 +359,8 @@ def model_logits_fast(ids, w, cfg, positions=None) -> torch.Tensor:
         g = fast_linear(x, w[p + "mlp.gate_proj.weight"])
         u = fast_linear(x, w[p + "mlp.up_proj.weight"])
         h = h + fast_linear(silu_and_mul(g, u), w[p + "mlp.down_proj.weight"])
+    if rows is not None:
+        h = h[torch.tensor(list(rows), dtype=torch.long)]
     h = rms_norm(h, w["model.norm.weight"], eps)
     head = w.get("lm_head.weight")
     if head is None:

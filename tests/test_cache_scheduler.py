@@ -138,11 +138,37 @@ def test_state_rows_are_zeroed_at_admission():
     model = structure("A")
     model.blocks[1].mixer.state_spec = lambda: StateSpec((3,), torch.float32)
     m = CacheManager(model, page_size=4, num_pages=4, max_requests=2, dtype=torch.float32, device="cpu")
-    assert m.layer(0).state is None and m.layer(1).state.shape == (2, 3)
+    # a row for each request slot and a spare one, which the rows that pad a graph's batch name
+    assert m.layer(0).state is None and m.layer(1).state.shape == (2 + 1, 3) and m.pad_slot == 2
     a = m.admit()
     m.layer(1).state[a] += 5.0
     m.release(a)
     assert m.admit() == a and float(m.layer(1).state[a].abs().sum()) == 0.0
+
+
+def test_padding_rows_stay_inside_every_per_slot_tensor():
+    """A decode batch filled up to a graph's size names the spare slot for its padding rows:
+    inside the block table of every group and inside every mixer's state rows."""
+    from litellmengine_amd.engine.batch import StepEntry, layout_step, views_of
+    from litellmengine_amd.parts import StateSpec
+
+    model = structure("C")
+    model.blocks[0].mixer.state_spec = lambda: StateSpec((5,), torch.float32)
+    m = CacheManager(model, page_size=4, num_pages=8, max_requests=3, dtype=torch.float32, device="cpu")
+    slots = [m.admit() for _ in range(3)]
+    m.extend_many([(s, 1) for s in slots])
+    for pad_to, entries in ((8, [StepEntry(s, [1], [0]) for s in slots]), (4, [])):  # the second: a warm-up batch
+        layout = layout_step(entries, m, all_rows=True, pad_to=pad_to)
+        v = views_of(layout.host, layout.sizes())
+        seq_slots, kv_lens = v[3], v[5]
+        assert layout.num_seqs == pad_to and int(seq_slots.max()) == m.pad_slot
+        assert all(int(seq_slots.max()) < g.block_table.shape[0] for g in m.groups)
+        assert all(int(seq_slots.max()) < state.shape[0] for state in m.states.values())
+        pads = seq_slots == m.pad_slot
+        assert int(pads.sum()) == pad_to - len(entries) and bool((kv_lens[pads] == 1).all())
+        for g, mapping in zip(m.groups, v[7:]):
+            assert bool((mapping[len(entries):] == -1).all())  # nothing is written for them
+            assert int(g.block_table[m.pad_slot, 0]) == g.pool.num_pages  # the page that is never handed out
 
 
 @pytest.mark.parametrize("which,seed", [("A", 0), ("A", 1), ("C", 2), ("C", 3)])

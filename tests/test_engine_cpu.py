@@ -100,3 +100,50 @@ def test_a_cache_record_that_is_no_key_value_pair_on_the_cpu(monkeypatch):
     monkeypatch.setattr(parts_tests, "make_context",
                         lambda dtype: BuildContext(dtype=dtype, device=torch.device("cpu"), ops=TorchOps()))
     parts_tests.test_a_cache_record_that_is_no_key_value_pair(torch.float32)
+
+
+def test_every_group_has_a_page_size_and_a_pool_of_its_own(tmp_path):
+    """Tiny C has layers with a window of 20 beside layers that see everything: two groups.
+    The windowed group gets pages of 4 tokens and a pool sized by its window, the other pages
+    of 16 and the whole capacity; the logits do not change, and a request four times as long
+    as the windowed pool fits."""
+    from litellmengine_amd.cache import GroupSizes
+    from litellmengine_amd.engine import LLMEngine
+
+    d = make_model_dir(tmp_path, "C")
+    cfg, w = plain.read_model_dir(d)
+    model = load_model(d, torch.float32, device="cpu", ops=TorchOps())
+    specs = {m.cache_spec() for m in model.cache_layers().values()}
+    windowed = next(s for s in specs if s.window is not None)
+    cache = CacheManager(model, page_size=16, num_pages=12, max_requests=2, dtype=torch.float32, device="cpu",
+                         max_tokens_per_step=9, group_sizes={windowed: GroupSizes(page_size=4)})
+    by_window = {g.window: g for g in cache.groups}
+    assert by_window[None].page_size == 16 and by_window[None].pool.num_pages == 12
+    # 20 - 1 + 9 positions in pages of 4, wherever they start: 8 pages a request
+    assert by_window[20].page_size == 4 and by_window[20].pool.num_pages == 2 * 8
+    assert by_window[20].max_pages_per_request == 12 * 16 // 4  # the table still covers the longest request
+    runner = ModelRunner(model, cache)
+    tokens = random_tokens(150, cfg["vocab_size"], 17)
+    want = plain.model_logits_fast(tokens, w, cfg)
+    got = run_cut(runner, tokens, [9, 2, 7, 9, 1, 1, 8] + [9] * 12 + [5])
+    assert (got.double() - want).abs().max().item() < 2e-5
+    assert all(g.pool.num_held == 0 for g in cache.groups)
+
+    # through the engine: the windowed pool is sized from the scheduler's budget
+    engine = LLMEngine(model, page_size=8, num_pages=40, max_requests=3, max_tokens_per_step=12)
+    sizes = {g.window: (g.page_size, g.pool.num_pages) for g in engine.cache.groups}
+    assert sizes[None] == (8, 40) and sizes[20] == (8, 3 * (-(-(19 + 12) // 8) + 1))
+    prompts = [random_tokens(n, cfg["vocab_size"], 80 + i) for i, n in enumerate((70, 33, 90))]
+    out = engine.generate(prompts, 12)
+    for p, o in zip(prompts, out):
+        assert o == plain.generate_greedy(p, w, cfg, 12)
+    assert engine.scheduler.num_preemptions == 0 and all(g.pool.num_held == 0 for g in engine.cache.groups)
+
+
+def test_a_mixer_may_ask_for_its_own_page_size():
+    from litellmengine_amd.parts.base import KVCacheSpec
+
+    assert KVCacheSpec(2, 16, None, 32).page_size == 32
+    assert KVCacheSpec(2, 16) != KVCacheSpec(2, 16, page_size=32)  # another page size: another group
+    with pytest.raises(ValueError):
+        KVCacheSpec(2, 16, page_size=0)

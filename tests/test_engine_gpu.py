@@ -206,6 +206,12 @@ ODD = [
     # head size 96 (matrix cores, three 32-element steps), group of 3, page size 48
     dict(num_hidden_layers=2, hidden_size=96, num_attention_heads=6, num_key_value_heads=2, head_dim=96,
          intermediate_size=136, vocab_size=257, rope_theta=5e5, rms_norm_eps=1e-6, tie_word_embeddings=True, page=48),
+    # a group of 16: one decoded token fills the 16-row tile of the decode kernels exactly; heads of 128
+    dict(num_hidden_layers=2, hidden_size=72, num_attention_heads=32, num_key_value_heads=2, head_dim=128,
+         intermediate_size=104, vocab_size=211, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, page=16),
+    # a group of 32 on one kv head: a decoded token has more rows than a tile, so it goes the prompt kernels' way
+    dict(num_hidden_layers=2, hidden_size=88, num_attention_heads=32, num_key_value_heads=1, head_dim=64,
+         intermediate_size=120, vocab_size=197, rope_theta=2e5, rms_norm_eps=1e-5, tie_word_embeddings=True, page=16),
 ]
 
 

@@ -217,6 +217,7 @@ def test_which_products_are_taken_in_slices():
     assert o.slices_for(128, n, 4096) == 4 and o.slices_for(16, n, 4096) == 0 and o.slices_for(129, n, 4096) == 0
     assert o.slices_for(64, 64 * units, 4096) == 0      # wide: rows enough for every CU
     assert o.slices_for(64, n + 8, 4096) == 0           # no multiple of 64 rows
+    assert o.slices_for(64, 8192 + 64, 32768) == 0      # wider than the norm that adds the slices up takes
     assert o.slices_for(64, n, 4096 + 256) == 0         # no whole slices
     if units == 256:
         # a long K beside few rows (down_proj of the 32B and 14B sizes): slices although the workgroups fill
@@ -226,7 +227,7 @@ def test_which_products_are_taken_in_slices():
     x = rnd((40, 4096), torch.bfloat16, 65)
     w = rnd((n, 4096), torch.bfloat16, 66, 0.05)
     assert o.linear(x, w).shape == (40, n)                       # a caller that said nothing gets the product
-    assert o.linear(x, w, sums_ok=True).shape == (4, 40, n)      # a delta of the residual stream may come in slices
+    assert o.linear(x, w, sums_ok=True).sums.shape == (4, 40, n)  # a delta of the residual stream may come in slices
 
 
 @pytest.mark.parametrize("K", [1024, 2048, 3072, 4096, 5120, 6144, 8192])
@@ -444,7 +445,10 @@ def test_paged_attention(dtype, nq, nkv, d, P, window):
 
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 16, 16, None), (16, 2, 64, 32, None),
                                                (6, 1, 48, 16, 40), (2, 1, 256, 16, None), (32, 8, 128, 16, 700),
-                                               (3, 1, 160, 48, None), (5, 5, 80, 16, 9)])
+                                               (3, 1, 160, 48, None), (5, 5, 80, 16, 9),
+                                               # groups of 16 and 32: a decoded token fills a tile, or is more than one
+                                               (32, 2, 128, 16, None), (32, 1, 64, 16, None), (32, 1, 128, 32, 300),
+                                               (32, 2, 64, 16, None)])
 @pytest.mark.parametrize("lens", [
     [(0, 9), (17, 1), (30, 2), (5, 11)],          # portions beside decoded tokens
     [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
@@ -480,7 +484,10 @@ def test_float32_matrix_core_attention(nq, nkv, d, P, window, lens):
 
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(8, 2, 128, 16, None), (4, 4, 32, 16, None), (16, 2, 64, 32, None),
                                                (6, 1, 96, 16, 40), (8, 2, 256, 16, None), (32, 8, 128, 16, 700),
-                                               (3, 1, 160, 48, None), (8, 2, 128, 48, None), (4, 1, 128, 32, 100)])
+                                               (3, 1, 160, 48, None), (8, 2, 128, 48, None), (4, 1, 128, 32, 100),
+                                               # groups of 16 and 32: a decoded token fills a tile, or is more than one
+                                               (32, 2, 128, 16, None), (32, 1, 64, 16, None), (32, 1, 128, 32, 300),
+                                               (32, 2, 64, 16, None), (48, 1, 32, 16, None)])
 @pytest.mark.parametrize("lens", [
     [(0, 9), (17, 1), (30, 2), (5, 11)],          # portions beside decoded tokens
     [(1999, 1), (640, 1), (31, 1), (0, 1)],       # decoding only, long contexts: key splits
@@ -515,7 +522,8 @@ def test_matrix_core_attention(nq, nkv, d, P, window, lens):
 
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32, None])
 @pytest.mark.parametrize("nq,nkv,d,P,window", [(32, 8, 128, 16, None), (4, 4, 64, 32, None), (16, 2, 64, 16, 50),
-                                               (6, 1, 192, 48, None), (8, 2, 256, 16, 900)])
+                                               (6, 1, 192, 48, None), (8, 2, 256, 16, 900),
+                                               (32, 2, 128, 16, None), (16, 1, 64, 16, 1100)])  # a group of 16: one token a tile
 @pytest.mark.parametrize("lens", [
     [(1999, 1), (640, 1), (31, 1), (0, 1)],   # long contexts: the new key lies in the last of several key splits
     [(15, 1), (16, 1), (47, 1)],              # the new key is the last of a page / the first of a new one

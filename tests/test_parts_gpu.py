@@ -401,3 +401,81 @@ def test_a_cache_record_that_is_no_key_value_pair(dtype):
         assert cache.groups[1].pool.num_held <= (window + page - 1) // page + 1  # the window let pages go
         runner.release(slot)
     assert all(g.pool.num_held == 0 for g in cache.groups)
+
+
+# ---------------------------------------------------------------------------------------
+# a mixer with state of its own that decodes through captured graphs
+# ---------------------------------------------------------------------------------------
+class GraphSafeRunningMean(RunningMeanMixer):
+    """The running mean again, from the step's device arrays alone (no host-side view of the
+    batch), so that decode steps may be captured and replayed.  Every run of forward() advances
+    the state: a capture that ran a request's step more than once would count its token twice."""
+
+    graph_safe = True
+
+    def forward(self, x, step, cache):
+        seq = step.token_seq.long()                      # [N] request of each token, within this batch
+        rows = step.seq_slots.long()                     # [S] state row of each request (padding: the spare row)
+        first = step.cu_tokens.long()[:-1]               # [S] first token of each request
+        xf = x.float()
+        run = torch.cumsum(xf, dim=0)
+        before = torch.cat([torch.zeros_like(run[:1]), run])[first]  # [S, H] sum of the tokens before each request
+        state = cache.state[rows]                        # [S, H + 1]
+        sums = state[seq, :-1] + run - before[seq]
+        index = torch.arange(x.shape[0], device=x.device)
+        counts = state[seq, -1] + (index - first[seq] + 1).float()
+        last = step.cu_tokens.long()[1:] - 1
+        cache.state[rows] = torch.cat([sums[last], counts[last, None]], dim=1)
+        return self.ctx.ops.linear((sums / counts[:, None]).to(x.dtype), self.weight)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_mixer_with_state_decodes_through_graphs(dtype):
+    """Two requests: prompts in portions, then fifteen single tokens each through captured
+    graphs (two batch buckets: the second request ends first), against the running mean computed
+    whole and against the same steps without graphs.  The state of a request moves once per step:
+    the runs that warm a graph's kernels up before its capture touch the spare state row only."""
+    hidden, vocab = 40, 61
+    outs = {}
+    for use_graphs in (True, False):
+        block = PreNormBlock(RMSNorm("l0.n1", hidden, 1e-5), GraphSafeRunningMean("l0.mean.weight", hidden),
+                             RMSNorm("l0.n2", hidden, 1e-5), GatedMLP("l0.mlp.", hidden, 56))
+        model = one_block_model(block, hidden, vocab)
+        ctx, w = bound(model, dtype, seed=6)
+        model.ctx = ctx
+        cache = CacheManager(model, page_size=16, num_pages=4, max_requests=3, dtype=dtype, device=ctx.device)
+        assert cache.states[0].shape == (3 + 1, hidden + 1)  # a spare row for the rows that pad a batch
+        runner = ModelRunner(model, cache, use_graphs=use_graphs)
+        assert runner.use_graphs == use_graphs
+        seqs = [random_tokens(30, vocab, 11), random_tokens(22, vocab, 12)]
+        slots = [runner.admit(), runner.admit()]
+        got = [[], []]
+        got[0].append(runner.step([StepEntry(slots[0], seqs[0][:9], list(range(9)))]))
+        out = runner.step([StepEntry(slots[0], seqs[0][9:15], list(range(6))), StepEntry(slots[1], seqs[1][:7], list(range(7)))])
+        got[0].append(out[:6])
+        got[1].append(out[6:])
+        at = [15, 7]
+        while at[0] < 30:
+            live = [i for i in (0, 1) if at[i] < len(seqs[i])]
+            out = runner.step([StepEntry(slots[i], [seqs[i][at[i]]], [0]) for i in live])
+            for n, i in enumerate(live):
+                got[i].append(out[n : n + 1].clone())
+                at[i] += 1
+        if use_graphs:
+            assert runner.num_captures == 2, "batches of two and of one: two graphs"
+        outs[use_graphs] = [torch.cat(g).cpu().double() for g in got]
+
+    def whole(ids):
+        T = len(ids)
+        x = plain.embedding(ids, w["e.weight"])
+        m = torch.cumsum(plain.rms_norm(x, w["l0.n1"], 1e-5), 0) / torch.arange(1, T + 1, dtype=D)[:, None]
+        r = x + plain.linear(m, w["l0.mean.weight"])
+        r = r + plain.gated_mlp(plain.rms_norm(r, w["l0.n2"], 1e-5), w["l0.mlp.gate_proj.weight"],
+                                w["l0.mlp.up_proj.weight"], w["l0.mlp.down_proj.weight"])
+        return plain.fast_linear(plain.rms_norm(r, w["fn.weight"], 1e-6), w["head.weight"])
+
+    for i, ids in enumerate(seqs):
+        want = whole(ids)
+        for use_graphs in (True, False):
+            err = (outs[use_graphs][i] - want).abs().max().item()
+            assert err < TOL[dtype], (i, use_graphs, err)

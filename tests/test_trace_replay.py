@@ -170,3 +170,61 @@ def test_trace_qwen3_8b_layer_sizes_mixed(tmp_path, model_dirs_8b, sharp, dtype)
     tol = PEAK_8B[dtype][1] if sharp else TOL_8B[dtype]
     worst = check_dumps(out, tb, want, tol)
     print(f"8B-size mixed trace {dtype} sharp={sharp}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")
+
+
+class SomeRows:
+    """The plain model's logits at some positions of a request, indexed by position
+    (what check_dumps asks of the expected logits of a request)."""
+
+    def __init__(self, positions, logits):
+        self.at = {int(p): i for i, p in enumerate(positions)}
+        self.logits = logits
+        self.shape = (max(self.at) + 1, logits.shape[1])
+
+    def __getitem__(self, pos):
+        return self.logits[self.at[int(pos)]]
+
+
+_long_oracle = {}
+
+
+def long_trace_oracle(d, long_ids, short_ids, wanted):
+    """The plain model in float64 at the wanted positions (the head runs on those rows only);
+    made once for both dtypes."""
+    from tests.plain import qwen3_plain as plain
+
+    if d not in _long_oracle:
+        pcfg, w = plain.read_model_dir(d, dtype=torch.float64)
+        _long_oracle[d] = {rid: SomeRows(wanted[rid], plain.model_logits_fast(ids, w, pcfg, rows=wanted[rid]))
+                           for rid, ids in (("long", long_ids), ("short", short_ids))}
+    return _long_oracle[d]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_qwen3_8b_layer_sizes_across_4096(tmp_path, model_dirs_8b, dtype):
+    """A request of 4200 tokens at the 8B layer sizes: most of it in two portions, then token by
+    token from position 4056 to the end, across the context of 4096 at which the benchmark runs
+    (sixteen key splits at batch 1) and across the table's 256th page; a short request decodes
+    beside it for a while (another batch bucket), and is ended so that its pages are used again."""
+    d, requests, _, _ = model_dirs_8b(False)
+    vocab = QWEN3_8B_LAYERS["vocab_size"]
+    long_ids, short_ids = random_tokens(4200, vocab, 31), random_tokens(120, vocab, 32)
+    head = 4056
+    tb = TraceBuilder()
+    tb.step([("long", long_ids[:2048], [0, 2047])])
+    tb.step([("long", long_ids[2048:head], [0, head - 2049]), ("short", short_ids[:70], [69])])
+    for i in range(head, len(long_ids)):
+        entries = [("long", [long_ids[i]], [0])]
+        j = 70 + (i - head)
+        if j < len(short_ids):
+            entries.append(("short", [short_ids[j]], [0]))
+        last_short = j == len(short_ids) - 1
+        tb.step(entries, end=(["short"] if last_short else []) + (["long"] if i == len(long_ids) - 1 else []))
+    wanted = {"long": sorted({pos for rows in tb.rows.values() for rid, pos in rows if rid == "long"}),
+              "short": sorted({pos for rows in tb.rows.values() for rid, pos in rows if rid == "short"})}
+    want = long_trace_oracle(d, long_ids, short_ids, wanted)
+    out = str(tmp_path / "out")
+    run_tool(d, dtype, out, tb, page_size=16)
+    worst = check_dumps(out, tb, want, TOL_8B[dtype])
+    print(f"8B-size trace across 4096 {dtype}: worst relative error {worst:.3g}, pool {tb.max_tokens} tokens")

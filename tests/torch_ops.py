@@ -26,7 +26,19 @@ class TorchOps:
     def embedding(self, ids, table):
         return table[ids.long()].to(torch.float32)
 
+    # the fused and sliced forms are the HIP kernels' own: this stand-in offers none of them
+    def can_fold_norm(self, rows, width, dtype):
+        return False
+
+    def can_fuse_rope_attention(self, *sizes):
+        return False
+
+    def slices_for(self, M, N, K):
+        return 0
+
     def add_rmsnorm(self, hidden, delta, weight, eps, out_dtype, rows=None):
+        if hasattr(delta, "sums"):  # parts.base.PartialSums
+            delta = delta.sums
         if delta is not None and delta.dim() == 3:  # partial sums of a product taken in slices
             delta = delta.to(self.cd).sum(0)
         if rows is None:
@@ -46,7 +58,8 @@ class TorchOps:
         y = xx / torch.sqrt((xx * xx).mean(-1, keepdim=True) + eps) * weight.to(self.cd)
         return y.to(x.dtype)
 
-    def linear(self, x, weight, out_dtype=None):
+    def linear(self, x, weight, out_dtype=None, fold=None, sums_ok=False):
+        assert fold is None, "this stand-in folds no norm (can_fold_norm says so)"
         return (x.to(self.cd) @ weight.to(self.cd).t()).to(out_dtype or x.dtype)
 
     def rope_table(self, positions, inv_freq):
