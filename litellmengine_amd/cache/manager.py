@@ -318,6 +318,17 @@ class CacheManager:
     def extend(self, slot: int, new_len: int) -> None:
         self.extend_many([(slot, new_len)])
 
+    def shrink_many(self, wants: Sequence[Tuple[int, int]]) -> None:
+        """Undo an extend_many whose step did not happen: wants = [(slot, the length that is
+        committed), ...]; the pages beyond those lengths go back, last taken first."""
+        for slot, length in wants:
+            self._check_live(slot)
+            if length != self._length[slot]:
+                raise ValueError("a request shrinks back to its committed length only")
+        n, slots, lens, keep = self._arrays(wants)
+        for group in self.groups:
+            group._lib.lle_pt_shrink_many(group._h, n, slots, lens)
+
     def commit(self, slot: int, new_len: int) -> None:
         """The positions < new_len are now written; windows move on."""
         self._check_live(slot)

@@ -32,6 +32,8 @@ _SIGNATURES = {
     "lle_pt_grow": ([_P, _I, _I], _I),
     "lle_pt_pages_needed_many": ([_P, _I, _P, _P], _I),
     "lle_pt_grow_many": ([_P, _I, _P, _P], _I),
+    "lle_pt_shrink": ([_P, _I, _I], None),
+    "lle_pt_shrink_many": ([_P, _I, _P, _P], None),
     "lle_pt_trim": ([_P, _I, _I], None),
     "lle_pt_trim_many": ([_P, _I, _P, _P], None),
     "lle_pt_release_slot": ([_P, _I], None),

@@ -1562,10 +1562,19 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
                                          ws_stride, S, nq, nkv, P, page_stride, max_pages, window, scale_log2,
                                          nsplit_decode, fused, stream);
         }
-        if (e != 0) return e;
+        if (e != 0) {
+            if (lane) (void)hipStreamSynchronize(lane->stream);
+            return e;
+        }
     }
+    // After the fork an error may not leave the side stream running behind the caller's back: the
+    // caller frees `out` and the workspaces on its own stream, and the decode kernel still writes them.
     if (lane) {
-        if (hipEventRecord(lane->join, lane->stream) != hipSuccess) return (int)hipGetLastError();
+        if (hipEventRecord(lane->join, lane->stream) != hipSuccess) {
+            const int e = (int)hipGetLastError();
+            (void)hipStreamSynchronize(lane->stream);
+            return e;
+        }
         stream = prefill_stream;
     }
     if (run_prefill) {
@@ -1588,7 +1597,11 @@ static int launch_mfma(const bf16_t* q, bf16_t* kv_layer, const int32_t* block_t
             launch(std::integral_constant<int, PRE_RT_OF(DK)>{}, Four{});
         }
     }
-    if (lane && hipStreamWaitEvent(stream, lane->join, 0) != hipSuccess) return (int)hipGetLastError();
+    if (lane && hipStreamWaitEvent(stream, lane->join, 0) != hipSuccess) {
+        const int e = (int)hipGetLastError();
+        (void)hipStreamSynchronize(lane->stream);
+        return e;
+    }
     if (ws_stride > 1)  // a batch of one kind needs no look at the tokens' requests
         mfma_combine_kernel<<<dim3(N, nq), LLE_WAVE, 0, stream>>>(
             ws_o, ws_ml, ws_stride, cu_tokens, token_seq, out, nq, nkv, D, run_decode ? nsplit_decode : nsplit_prefill,

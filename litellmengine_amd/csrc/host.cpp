@@ -176,6 +176,35 @@ int lle_pt_grow_many(void* h, int n, const int32_t* slots, const int32_t* new_le
     return LLE_HOST_OK;
 }
 
+// A step that did not happen after all: the pages beyond those of `length` positions go back, last
+// taken first (after lle_pt_grow_many and lle_pt_shrink_many with the lengths of before, the stack
+// is what it was), and what was noted for the device table about them is dropped.
+void lle_pt_shrink(void* h, int slot, int length) {
+    PageTables* t = pt(h);
+    std::vector<int32_t>& table = t->tables[slot];
+    const int keep = std::max(t->pages_for(std::max(length, 0)), t->first_live[slot]);
+    if ((int)table.size() <= keep) return;
+    while ((int)table.size() > keep) {
+        if (table.back() >= 0) t->give_back(table.back());
+        table.pop_back();
+    }
+    const int row = slot * t->max_pages_per_request;
+    size_t out = 0;
+    for (size_t i = 0; i < t->pending_index.size(); ++i) {
+        const int32_t at = t->pending_index[i];
+        if (at >= row + keep && at < row + t->max_pages_per_request) continue;
+        t->pending_index[out] = at;
+        t->pending_page[out] = t->pending_page[i];
+        ++out;
+    }
+    t->pending_index.resize(out);
+    t->pending_page.resize(out);
+}
+
+void lle_pt_shrink_many(void* h, int n, const int32_t* slots, const int32_t* lengths) {
+    for (int i = n - 1; i >= 0; --i) lle_pt_shrink(h, slots[i], lengths[i]);
+}
+
 // With a window w the next query (position `length`) sees keys >= length - w + 1: the pages
 // before that one's are given back.
 void lle_pt_trim(void* h, int slot, int length) {

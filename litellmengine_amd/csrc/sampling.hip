@@ -171,6 +171,13 @@ __device__ __forceinline__ float wave_inclusive_scan(float v, int lane) {
     return v;
 }
 
+// The weight of one id.  A logit that is no number (or an infinite one beside an infinite
+// maximum) has none: it is never picked and moves no other id's share of the running sum.
+__device__ __forceinline__ float sample_weight(float logit, float big, float inv_t) {
+    const float e = expf((logit - big) * inv_t);
+    return e == e ? e : 0.f;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits,
                                                                      const float* __restrict__ temperature,
                                                                      const float* __restrict__ uniform,
@@ -224,7 +231,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
             }
 #pragma unroll
             for (int j = 0; j < SAMPLE_LINE / LLE_WAVE; ++j)
-                part += base + lane + LLE_WAVE * j < V ? expf((v[j] - big) * inv_t) : 0.f;
+                part += base + lane + LLE_WAVE * j < V ? sample_weight(v[j], big, inv_t) : 0.f;
         }
         part = wave_sum(part);
         if (lane == 0) s_seg[seg] = part;
@@ -278,7 +285,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     }
     __syncthreads();
     const int seg = s_seg_pick;
-    if (seg < 0) {  // no id has weight (a row of NaN): the greedy pick
+    if (seg < 0) {  // no id has weight (a row of NaN, or an infinite maximum): the greedy pick
         if (t == 0) out[blockIdx.x] = s_big_i;
         return;
     }
@@ -288,7 +295,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         const int64_t base = ((int64_t)seg * per_seg + g) * SAMPLE_LINE;
         if (base >= V) break;
         const int64_t i = base + t;
-        const float p = i < V ? expf((row[i] - big) * inv_t) : 0.f;
+        const float p = i < V ? sample_weight(row[i], big, inv_t) : 0.f;
         const float inclusive = wave_inclusive_scan(p, lane);
         if (lane == LLE_WAVE - 1) s_wave[wave] = inclusive;
         __syncthreads();

@@ -119,18 +119,26 @@ class ModelRunner:
         """Run the entries as one batch.  Returns float32 logits [wanted, vocab] in
         the order of the entries and of their `want`.  Raises cache.OutOfPages,
         with nothing changed, when the pages for this step are not there.  With
-        `borrow` the result may alias memory that the next step overwrites."""
+        `borrow` the result may alias memory that the next step overwrites.
+        If the model raises (a kernel that refuses its operands), the step did not
+        happen: the pages it took go back and no length moves, so the same entries
+        can be stepped again (what a mixer keeps as state of its own is its own to mend)."""
         self.check(entries)
         cache = self.cache
-        wants = [(e.slot, cache.length(e.slot) + len(e.tokens)) for e in entries]
+        before = [(e.slot, cache.length(e.slot)) for e in entries]
+        wants = [(slot, length + len(e.tokens)) for (slot, length), e in zip(before, entries)]
         self.check_tokens(entries)
         cache.extend_many(wants)
-        if self.use_graphs and len(entries) <= self.MAX_GRAPH_BATCH and all(len(e.tokens) == 1 for e in entries):
-            logits = self._graph_step(entries, borrow)
-        else:
-            state = build_step(entries, cache, self.device, self.vocab_size)
-            self.last_step = state
-            logits = self.model.forward(state, cache)
+        try:
+            if self.use_graphs and len(entries) <= self.MAX_GRAPH_BATCH and all(len(e.tokens) == 1 for e in entries):
+                logits = self._graph_step(entries, borrow)
+            else:
+                state = build_step(entries, cache, self.device, self.vocab_size)
+                self.last_step = state
+                logits = self.model.forward(state, cache)
+        except BaseException:
+            cache.shrink_many(before)
+            raise
         cache.commit_many(wants)
         return logits
 

@@ -148,6 +148,7 @@ class Scheduler:
         r.cached_len = 0
         r.keep_session = False
         r.status = RequestStatus.FINISHED
+        self._last_served.pop(request_id, None)
 
     def _evict_parked(self) -> bool:
         """Take the cache of the session parked longest; False if none is parked."""
@@ -181,13 +182,20 @@ class Scheduler:
         budget = self.max_tokens_per_step
         chosen = None if only is None else set(only)
         mine = [r for r in self.running if chosen is None or r.request_id in chosen]
-        decoding = sorted((r for r in mine if r.extend_len == 1), key=lambda r: self._last_served.get(r.request_id, -1))
-        order = decoding + [r for r in mine if r.extend_len > 1]
+        turn = lambda r: self._last_served.get(r.request_id, -1)
+        decoding = sorted((r for r in mine if r.extend_len == 1), key=turn)
+        prompts = [r for r in mine if r.extend_len > 1]
+        # Decoders that alone fill the budget, step after step, would leave prompt tokens (of running
+        # requests and of waiting ones) standing until they finish: then a quarter of the budget is
+        # kept back from them (a budget of one token cannot be shared: decoders first).
+        others = bool(prompts) or any(chosen is None or w.request_id in chosen for w in self.waiting)
+        kept_back = max(1, budget // 4) if others and len(decoding) >= budget > 1 else 0
         plan: List[Portion] = []
-        for r in order:
-            if budget == 0:
-                break
-            n = min(r.extend_len, self.prefill_chunk, budget)
+        for r in decoding + prompts:
+            left = budget - kept_back if r.extend_len == 1 else budget
+            if left <= 0:
+                continue
+            n = min(r.extend_len, self.prefill_chunk, left)
             plan.append(Portion(r, r.cached_len, n, n == r.extend_len))
             budget -= n
 
@@ -242,6 +250,7 @@ class Scheduler:
 
     def _preempt(self, r: Request) -> None:
         self.cache.release(r.slot)
+        self._last_served.pop(r.request_id, None)  # when it runs again it counts as newly served
         r.slot = -1
         r.cached_len = 0
         r.status = RequestStatus.WAITING

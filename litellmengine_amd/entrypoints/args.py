@@ -19,7 +19,8 @@ class _Parser(argparse.ArgumentParser):
 
 def build_parser() -> argparse.ArgumentParser:
     p = _Parser(prog="litellmengine", add_help=True, allow_abbrev=False,
-                description="Generate tokens with a Qwen3 model on one MI355X.")
+                description="Generate tokens with the model in a folder (its config.json names the architecture) "
+                            "on one MI355X.")
     p.add_argument("--model", required=True, help="local model folder (config.json + safetensors)")
     p.add_argument("--prompt", default="What is the capital of France?", help="input prompt (needs tokenizer.json)")
     p.add_argument("--input-ids", "--prompt-ids", dest="input_ids", default=None,

@@ -36,7 +36,7 @@ def run(argv=None) -> int:
     args = parse_args(argv)
     device = resolve_device(args.device)
     out = sys.stdout
-    print("LiteLLMEngine (MI355X)", file=out)
+    print("litellmengine_amd (one MI355X)", file=out)
     print(f"Device: {device}", file=out)
     print("Config:", file=out)
     for label, value in (

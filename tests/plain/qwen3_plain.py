@@ -285,12 +285,19 @@ def generate_greedy(ids: Sequence[int], w, cfg, max_new: int, eos: int = -1) -> 
 # a vectorised twin of model_logits (same formulas, library products) used for
 # long sequences; test_plain.py checks it against the loop version above
 # --------------------------------------------------------------------------
-def _rope_fast(x, positions, theta):
+def _rope_fast(x, positions, theta, float32_angles=False):
+    """`float32_angles`: the angle as the reference forms it, a float32 product of the position and
+    a float32 frequency (src/layers/rotary.cu:81-83, :96-99).  At position p that product is off by
+    up to p * 2^-24 radians from the exact angle, which far into a long sequence is more than all
+    other rounding of a float32 run together; tests at thousands of positions compare like with like."""
     T, heads, d = x.shape
     half = d // 2
     i = torch.arange(half, dtype=torch.float64)
     inv_freq = theta ** (-(2.0 * i) / d)
-    ang = torch.tensor(list(positions), dtype=torch.float64)[:, None] * inv_freq[None, :]
+    if float32_angles:
+        ang = (torch.tensor(list(positions), dtype=torch.float32)[:, None] * inv_freq.float()[None, :]).double()
+    else:
+        ang = torch.tensor(list(positions), dtype=torch.float64)[:, None] * inv_freq[None, :]
     c = torch.cos(ang).to(x.dtype)[:, None, :]
     s = torch.sin(ang).to(x.dtype)[:, None, :]
     x1, x2 = x[..., :half], x[..., half:]
@@ -336,9 +343,10 @@ def first_layer_attention_probs(ids, w, cfg) -> torch.Tensor:
     return torch.softmax(scores.masked_fill(~allowed[None], float("-inf")), dim=-1)
 
 
-def model_logits_fast(ids, w, cfg, positions=None, rows=None) -> torch.Tensor:
+def model_logits_fast(ids, w, cfg, positions=None, rows=None, float32_angles=False) -> torch.Tensor:
     """`rows`: only these positions go through the final norm and the head (long sequences,
-    wide vocabularies); the result then has one row for each of them, in their order."""
+    wide vocabularies); the result then has one row for each of them, in their order.
+    `float32_angles`: see _rope_fast."""
     T = len(ids)
     positions = list(range(T)) if positions is None else positions
     nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -351,8 +359,8 @@ def model_logits_fast(ids, w, cfg, positions=None, rows=None) -> torch.Tensor:
         q = fast_linear(x, w[p + "self_attn.q_proj.weight"]).reshape(T, nq, d)
         k = fast_linear(x, w[p + "self_attn.k_proj.weight"]).reshape(T, nkv, d)
         v = fast_linear(x, w[p + "self_attn.v_proj.weight"]).reshape(T, nkv, d)
-        q = _rope_fast(rms_norm(q, w[p + "self_attn.q_norm.weight"], eps), positions, theta)
-        k = _rope_fast(rms_norm(k, w[p + "self_attn.k_norm.weight"], eps), positions, theta)
+        q = _rope_fast(rms_norm(q, w[p + "self_attn.q_norm.weight"], eps), positions, theta, float32_angles)
+        k = _rope_fast(rms_norm(k, w[p + "self_attn.k_norm.weight"], eps), positions, theta, float32_angles)
         a = _attention_fast(q, k, v, windows[i]).reshape(T, nq * d)
         h = h + fast_linear(a, w[p + "self_attn.o_proj.weight"])
         x = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)

@@ -186,6 +186,23 @@ def test_random_orders_lose_no_page(which, seed):
             slot = rng.choice(list(live))
             new_len = live[slot] + rng.randint(1, 9)
             if m.can_extend([(slot, new_len)]):
+                if rng.random() < 0.3:
+                    # a step that does not happen after all: grown with another request, then given back
+                    other = rng.choice(list(live))
+                    wants = [(slot, new_len)] + ([(other, live[other] + 5)] if other != slot else [])
+                    if m.can_extend(wants):
+                        stacks = [(g.pool.num_free, [g.tables[s] for s in live]) for g in m.groups]
+                        m.extend_many(wants)
+                        m.shrink_many([(s, live[s]) for s, _ in wants])
+                        assert [(g.pool.num_free, [g.tables[s] for s in live]) for g in m.groups] == stacks
+                        again = [g.pool.num_free for g in m.groups]
+                        m.extend_many(wants)  # ... and the pages come in the same order when it is tried again
+                        took = [[g.tables[s] for s, _ in wants] for g in m.groups]
+                        m.shrink_many([(s, live[s]) for s, _ in wants])
+                        m.extend_many(wants)
+                        assert [[g.tables[s] for s, _ in wants] for g in m.groups] == took
+                        m.shrink_many([(s, live[s]) for s, _ in wants])
+                        assert [g.pool.num_free for g in m.groups] == again
                 m.extend(slot, new_len)
                 m.commit(slot, new_len)
                 live[slot] = new_len
@@ -347,6 +364,35 @@ def test_decoders_take_turns_when_the_budget_is_below_their_number():
         assert window >= {r for r in ids if not s.requests[r].finished or r in window}
     counts = {r: sum(r in step for step in served[:5]) for r in ids}
     assert max(counts.values()) - min(counts.values()) <= 1, counts
+
+
+def test_prompts_are_not_starved_by_decoders_that_fill_the_budget():
+    """Six decoders and a budget of four tokens: a request that arrives with a prompt of ten
+    tokens is admitted at once and gets a share of every step, beside decoders that still take
+    turns; and what is released or preempted leaves nothing behind in the turn-taking record."""
+    s = Scheduler(manager(page_size=4, num_pages=64, max_requests=8), max_tokens_per_step=32)
+    decoders = [s.add_request([1, 2, 3], 30) for _ in range(6)]
+    run_plan(s, s.schedule())
+    assert all(r.extend_len == 1 for r in decoders)
+    s.max_tokens_per_step = 4
+    late = s.add_request(list(range(10)), 2)
+    seen = []
+    for step in range(16):
+        plan = s.schedule()
+        assert sum(p.num_tokens for p in plan) <= 4
+        seen.append([(p.request.request_id, p.num_tokens) for p in plan])
+        run_plan(s, plan)
+        if late.finished:
+            break
+    assert late.finished and step <= 12, seen  # ten steps for its prompt (a token each), two decoding
+    assert any(rid == late.request_id for rid, _ in seen[0]), "a share of the first step already"
+    assert all(sum(1 for rid, _ in plan if rid != late.request_id) >= 2 for plan in seen)  # decoders go on
+    # nothing of a released or a preempted request stays in the record
+    victim = decoders[0]
+    s.release_request(victim.request_id)
+    assert victim.request_id not in s._last_served
+    s._preempt(decoders[1])
+    assert decoders[1].request_id not in s._last_served and decoders[1].status is RequestStatus.WAITING
 
 
 def test_a_request_that_does_not_fit_leaves_parked_sessions_alone():

@@ -147,3 +147,42 @@ def test_a_mixer_may_ask_for_its_own_page_size():
     assert KVCacheSpec(2, 16) != KVCacheSpec(2, 16, page_size=32)  # another page size: another group
     with pytest.raises(ValueError):
         KVCacheSpec(2, 16, page_size=0)
+
+
+def test_a_step_that_fails_in_the_model_leaves_the_cache_as_it_was(tmp_path):
+    """A kernel error in the second layer of a step (the first layer has written its K and V by
+    then): pages, tables, lengths and what waits for the device table are what they were, and
+    the same entries stepped again give the plain model's logits."""
+    d = make_model_dir(tmp_path, "C")
+    cfg, w = plain.read_model_dir(d)
+    runner = make_runner(d, 4, 24)
+    cache, ops = runner.cache, runner.model.ctx.ops
+    a, b = random_tokens(30, cfg["vocab_size"], 3), random_tokens(11, cfg["vocab_size"], 4)
+    sa, sb = runner.admit(), runner.admit()
+    runner.step([StepEntry(sa, a[:13]), StepEntry(sb, b[:2])])
+
+    def snapshot():
+        return ([g.pool.num_free for g in cache.groups], [[g.tables[s] for s in (sa, sb)] for g in cache.groups],
+                [cache.length(sa), cache.length(sb)], [g.native.lib.lle_pt_num_pending(g.native.handle) for g in cache.groups])
+
+    before = snapshot()
+    calls, real = [0], ops.paged_attention
+
+    def failing(*args, **kw):
+        calls[0] += 1
+        if calls[0] == 2:
+            raise RuntimeError("the kernel refuses its operands")
+        return real(*args, **kw)
+
+    ops.paged_attention = failing
+    entries = [StepEntry(sa, a[13:30], list(range(17))), StepEntry(sb, b[2:11], list(range(9)))]
+    with pytest.raises(RuntimeError, match="refuses"):
+        runner.step(entries)
+    ops.paged_attention = real
+    assert snapshot() == before
+    got = runner.step(entries)
+    want = torch.cat([plain.model_logits_fast(a, w, cfg)[13:], plain.model_logits_fast(b, w, cfg)[2:]])
+    assert (got.double() - want).abs().max().item() < 2e-5
+    runner.release(sa)
+    runner.release(sb)
+    assert all(g.pool.num_held == 0 for g in cache.groups)

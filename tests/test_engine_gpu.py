@@ -235,3 +235,44 @@ def test_odd_sizes(tmp_path, index, dtype):
         got = run_cut(runner, tokens, cuts)
         err = (got.double() - want).abs().max().item() / max(1.0, want.abs().max().item())
         assert err < TOL[dtype], (cuts, err)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_kernel_error_in_the_middle_of_a_step_leaves_the_cache_consistent(tmp_path, dtype):
+    """The attention of the second layer refuses to launch (a KernelError, forced from the host)
+    after the first layer has written its keys and values: pages, tables and lengths are what
+    they were before the step, and the same entries stepped again match the plain model."""
+    from litellmengine_amd.csrc.ops import KernelError
+
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    cfg, w = plain.read_model_dir(d)
+    runner = make_runner(d, dtype, 8, 12)
+    cache, ops = runner.cache, runner.model.ctx.ops
+    a, b = random_tokens(40, cfg["vocab_size"], 3), random_tokens(19, cfg["vocab_size"], 4)
+    sa, sb = runner.admit(), runner.admit()
+    runner.step([StepEntry(sa, a[:21]), StepEntry(sb, b[:3])])
+    snapshot = lambda: ([g.pool.num_free for g in cache.groups], [[g.tables[s] for s in (sa, sb)] for g in cache.groups],
+                        [cache.length(sa), cache.length(sb)])
+    before = snapshot()
+    calls, real = [0], ops.paged_attention
+
+    def failing(*args, **kw):
+        calls[0] += 1
+        if calls[0] == 2:
+            raise KernelError("lle_paged_attention_mfma failed to launch: forced by the test")
+        return real(*args, **kw)
+
+    ops.paged_attention = failing
+    entries = [StepEntry(sa, a[21:40], list(range(19))), StepEntry(sb, b[3:19], list(range(16)))]
+    try:
+        with pytest.raises(KernelError):
+            runner.step(entries)
+    finally:
+        del ops.paged_attention  # the instance attribute: the class's method is back
+    assert calls[0] == 2 and snapshot() == before
+    got = runner.step(entries).cpu()
+    want = torch.cat([plain.model_logits_fast(a, w, cfg)[21:], plain.model_logits_fast(b, w, cfg)[3:]])
+    assert (got.double() - want).abs().max().item() < TOL[dtype]
+    runner.release(sa)
+    runner.release(sb)
+    assert all(g.pool.num_held == 0 for g in cache.groups)

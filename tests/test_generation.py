@@ -183,6 +183,42 @@ def test_temperature_generation_matches_plain_draw_by_draw_gpu(tmp_path):
                                                     max_tokens_per_step=24))
 
 
+@pytest.mark.gpu
+def test_temperature_generation_in_bfloat16_lands_where_the_plain_model_allows_gpu(tmp_path):
+    """The same workload in bfloat16.  The engine's logits are within 2e-2 of the plain model's,
+    so its running sum at temperature 0.7 is within 3 % of the plain one: the token it draws
+    must be one whose share of the plain running sum lies within that margin of the target, and
+    where the target is further than the margin from both ends of a token's share it must be
+    that token.  (A draw taken from the wrong row, the wrong uniform number or a wrong running
+    sum lands anywhere in the vocabulary: one chance in sixteen a draw to pass.)"""
+    d = make_model_dir(tmp_path, "B", dtype=torch.bfloat16)
+    model = load_model(d, "bfloat16")
+    eng = LLMEngine(model, page_size=8, num_pages=16, max_requests=4, prefill_chunk=16, max_tokens_per_step=24)
+    cfg, w = plain.read_model_dir(d)
+    prompts = [random_tokens(n, 503, 10 + i) for i, n in enumerate((1, 7, 23, 40))]
+    reqs = [eng.add_request(p, 6, temperature=0.7, seed=9) for p in prompts]
+    for r in reqs:
+        r.rng = RecordedDraws(r.rng)
+    eng.run_until_finished()
+    margin, decided = 0.03, 0
+    for r, p in zip(reqs, prompts):
+        assert len(r.generated) == 6 and len(r.rng.drawn) == 6
+        history = list(p)
+        for k, u in enumerate(r.rng.drawn):
+            row = plain.model_logits_fast(history, w, cfg)[-1]
+            cdf = torch.cumsum(torch.softmax(row.double() / 0.7, dim=0), dim=0)
+            got = r.generated[k]
+            lo, hi = (float(cdf[got - 1]) if got else 0.0), float(cdf[got])
+            assert lo - margin <= u <= hi + margin, (r.request_id, k, got, u, lo, hi)
+            exact = plain.temperature_pick(row, 0.7, u)
+            elo, ehi = (float(cdf[exact - 1]) if exact else 0.0), float(cdf[exact])
+            if elo + margin < u < ehi - margin:
+                decided += 1
+                assert got == exact, (r.request_id, k)
+            history.append(got)
+    print(f"bfloat16 temperature: {decided} of 24 draws decided beyond the margin")
+
+
 def test_a_draw_that_rounds_to_one_is_kept_below_one():
     from litellmengine_amd.sampling import Sampler
 
@@ -241,9 +277,59 @@ def test_command_line_and_python_front(tmp_path, capsys):
                      "--max-tokens", "4", "--temperature", "0.7"]) == 0
     ids = parse_new_token_ids(capsys.readouterr().out)
     assert len(ids) == 4 and all(0 <= i < 503 for i in ids)
+    # the draws are the request's own (seeded): the same command gives the same tokens, another seed of the
+    # draws others, and they are not the greedy ones
+    assert cli.main(["--model", str(only), "--random-weights", "--seed", "3", "--input-ids", "1,2,3",
+                     "--max-tokens", "4", "--temperature", "0.7"]) == 0
+    assert parse_new_token_ids(capsys.readouterr().out) == ids
+    assert cli.main(["--model", str(only), "--random-weights", "--seed", "3", "--input-ids", "1,2,3",
+                     "--max-tokens", "4", "--temperature", "0"]) == 0
+    assert parse_new_token_ids(capsys.readouterr().out) != ids
     assert cli.main(["--model", d, "--input-ids", "1,2", "--max-tokens", "0"]) == 1
     assert "--max-tokens must be greater than 0" in capsys.readouterr().err
     assert cli.main(["--model", d, "--input-ids", "1,x"]) == 1
+
+
+@pytest.mark.gpu
+def test_text_front_in_process_and_through_the_command_line(tmp_path, capsys):
+    """run_prompt with a small word tokenizer written here: the chat template is applied, the
+    prompt's ids go to the engine in-process and, with --engine, to the command line as a child
+    process (whose `New token ids:` line is parsed); both print the plain model's greedy reply."""
+    import os
+
+    from tokenizers import Tokenizer, models, pre_tokenizers
+
+    from litellmengine_amd.entrypoints import run_prompt
+    from tests.trace_util import ROOT
+
+    d = make_model_dir(tmp_path, "A", dtype=torch.bfloat16)
+    words = ["[UNK]", "user", "assistant", "what", "is", "the", "capital", "of", "france"] + [f"w{i}" for i in range(200)]
+    tok = Tokenizer(models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = pre_tokenizers.Whitespace()
+    tok.add_special_tokens(["<|im_start|>", "<|im_end|>"])
+    tok.save(os.path.join(d, "tokenizer.json"))
+    cfg, w = plain.read_model_dir(d)
+    prompt = "what is the capital of france"
+    start, end = tok.token_to_id("<|im_start|>"), tok.token_to_id("<|im_end|>")
+    ids = [start, 1] + [3, 4, 5, 6, 7, 8] + [end, start, 2]  # the template's line ends are no words
+    assert tok.encode("<|im_start|>user\n" + prompt + "<|im_end|>\n<|im_start|>assistant\n", add_special_tokens=False).ids == ids
+    want = plain.generate_greedy(ids, w, cfg, 6, eos=end)
+    text = tok.decode(want, skip_special_tokens=True)
+    common = ["--model", d, "--prompt", prompt, "--max-tokens", "6", "--dtype", "float32", "--show-full-text"]
+    assert run_prompt.main(common) == 0
+    out = capsys.readouterr().out
+    assert f"prompt: {len(ids)} tokens\n  " + ",".join(map(str, ids)) in out
+    assert f"reply: {len(want)} tokens\n{text}\n" in out and "prompt and reply together:" in out
+    assert run_prompt.main(common + ["--engine", os.path.join(ROOT, "bin", "litellmengine")]) == 0
+    out = capsys.readouterr().out
+    assert "New token ids:" in out and f"reply: {len(want)} tokens\n{text}\n" in out
+    # without the template the words alone are the prompt
+    assert run_prompt.main(common[:-1] + ["--no-chat-template", "--eos-token-id", "999"]) == 0
+    out = capsys.readouterr().out
+    bare = plain.generate_greedy([3, 4, 5, 6, 7, 8], w, cfg, 6)
+    assert "prompt: 6 tokens\n  3,4,5,6,7,8" in out and tok.decode(bare, skip_special_tokens=True) in out
+    # an engine that fails hands its exit code on
+    assert run_prompt.main(common + ["--engine", "false"]) == 1
 
 
 def test_token_id_grammar_and_output_parsing():

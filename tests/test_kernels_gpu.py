@@ -663,3 +663,33 @@ def test_sample_every_region_of_the_row(V):
         if got[r] != want[r]:
             lo, hi = sorted((got[r], want[r]))
             assert hi - lo <= 2 and abs(float(cdf[r, hi - 1]) - float(u[r])) < 1e-5, (r, got[r], want[r])
+
+
+@pytest.mark.parametrize("V", [1500, 151936])
+def test_sample_skips_logits_that_are_no_numbers(V):
+    """NaN logits in the middle of a row (and a row with an infinite logit) get no weight: the
+    picks are those of the same row with the NaNs set to -inf, wherever the NaNs stand; a row
+    whose maximum is +inf is that id."""
+    g = torch.Generator().manual_seed(13)
+    R = 32
+    logits = (0.5 * torch.randn((R, V), generator=g))
+    bad = torch.randint(0, V, (R, 5), generator=g)
+    bad[:, 0] = V // 2  # one of them in the middle of every row
+    clean = logits.clone()
+    for r in range(R):
+        logits[r, bad[r]] = float("nan")
+        clean[r, bad[r]] = float("-inf")
+    temperature = torch.full((R,), 0.8)
+    u = ((torch.arange(R, dtype=torch.float64) + 0.41) / R).float()
+    o = ops()
+    got = o.sample(logits.cuda(), temperature.cuda(), u.cuda()).cpu().tolist()
+    same = o.sample(clean.cuda(), temperature.cuda(), u.cuda()).cpu().tolist()
+    assert got == same
+    p = torch.softmax(clean.double() / 0.8, dim=1)
+    cdf = torch.cumsum(p, dim=1)
+    want = torch.searchsorted(cdf, u.double().unsqueeze(1) * cdf[:, -1:], right=True).squeeze(1).tolist()
+    for r in range(R):
+        assert got[r] not in bad[r].tolist()
+        assert abs(got[r] - want[r]) <= 2 + 5, (r, got[r], want[r])  # a boundary's rounding, and the ids skipped
+    logits[3, 77] = float("inf")
+    assert o.sample(logits.cuda(), temperature.cuda(), u.cuda()).cpu().tolist()[3] == 77

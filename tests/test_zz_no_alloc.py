@@ -31,17 +31,25 @@ def test_static_argmax_equals_workspace_argmax_twice_in_a_row():
     dev = torch.device("cuda", torch.cuda.current_device())
     g = torch.Generator(device="cpu").manual_seed(5)
     stream = torch.cuda.current_stream().cuda_stream
+    # The library's code and its static array come to the device with its first launch; after that
+    # a call may not change what the device has free (torch's own counters cannot see a hipMalloc
+    # made inside the library: hipMemGetInfo, through mem_get_info, can).
+    warm = torch.zeros((2, 4099), device=dev)
+    assert static(warm.data_ptr(), torch.empty(2, dtype=torch.int32, device=dev).data_ptr(), 2, 4099, stream) == 0
+    torch.cuda.synchronize()
     # the second call is smaller in both directions: what the first left in the buffer must not show
     for rows, vocab in ((37, 151936), (5, 4099), (MAX_ROWS, 2048 * 3 + 17), (1, 7)):
         logits = torch.randn((rows, vocab), generator=g).to(dev)
         logits[0, vocab // 2] = logits[0, vocab - 1] = 50.0  # a tie: the first maximum wins
         want = ops.argmax(logits)
         out = torch.full((rows,), -7, dtype=torch.int32, device=dev)
-        before = torch.cuda.memory_allocated(dev)
+        torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
         code = static(logits.data_ptr(), out.data_ptr(), rows, vocab, stream)
         assert code == 0, lib.lle_error_string(code).decode()
-        assert torch.cuda.memory_allocated(dev) == before
         torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated(dev) == before
+        assert torch.cuda.mem_get_info(dev)[0] == free_before, "the call took device memory"
         assert torch.equal(out, want), (rows, vocab)
         assert out[0].item() == vocab // 2
         assert torch.equal(out.cpu().long(), logits.cpu().argmax(dim=1))
