@@ -13,7 +13,9 @@ A "step" is one decode step of the whole engine (scheduler, model step over the
 paged cache, sampling) with `batch` live requests whose context ends at
 `context` tokens.  Seeded random weights (bfloat16), uniform random token ids.
 One JSON line is printed: `value` = decoded tokens per second, `prefill` = a
-2048-token prompt in one step, `roofline` = bytes the decode step has to read
+2048-token prompt in one step, `more` = the same measurements, shorter, of the true 32-bit
+path, of the Qwen3-32B sizes and of the reference's own benchmark shape (default line only;
+--no-more skips them), `roofline` = bytes the decode step has to read
 (every weight it uses once + the cache of the live requests) / its time against
 8 TB/s, `points` = decode at batch 1 and 64.  Both rooflines are also given against
 what this machine reaches on kernels that do nothing else (`measured_peak`: a
@@ -178,10 +180,11 @@ def flat_config(cfg, full_layers, **more):
     return d
 
 
-def reference_workload(args):
+def time_reference_workload(dtype, runs, warmup):
     """The shape of the reference's benchmark (src/benchmark/generation_benchmark.cpp:259-315,
-    :430-526): 32 requests, 64-token prompts, 64 new tokens each, greedy; one warm-up run, then
-    the whole run is timed, prompts included; new tokens / wall-clock."""
+    :430-526): 32 requests, 64-token prompts, 64 new tokens each, greedy; warm-up runs, then
+    the whole run is timed, prompts included.  Returns (config, requests, prompt length, new
+    tokens, seconds a run)."""
     import torch
 
     from litellmengine_amd.config import Qwen3Config
@@ -189,13 +192,13 @@ def reference_workload(args):
     from litellmengine_amd.models import random_model
 
     cfg = Qwen3Config.from_dict(SIZES_0P6B)
-    model = random_model(cfg, seed=0, dtype=args.dtype)
+    model = random_model(cfg, seed=0, dtype=dtype)
     requests, prompt_len, new_tokens = 32, 64, 64
     pages_each = (prompt_len + new_tokens + PAGE_SIZE - 1) // PAGE_SIZE + 1
     engine = LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_each * requests, max_requests=requests,
                        max_tokens_per_step=requests * prompt_len, max_pages_per_request=pages_each)
     times = []
-    for run in range(args.warmup + args.steps):
+    for run in range(warmup + runs):
         prompts = random_prompts(requests, prompt_len, cfg.vocab_size, 1000 + run)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -203,9 +206,13 @@ def reference_workload(args):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         assert all(len(o) == new_tokens for o in out)
-        if run >= args.warmup:
+        if run >= warmup:
             times.append(dt)
-    dt = sum(times) / len(times)
+    return cfg, requests, prompt_len, new_tokens, sum(times) / len(times)
+
+
+def reference_workload(args):
+    cfg, requests, prompt_len, new_tokens, dt = time_reference_workload(args.dtype, args.steps, args.warmup)
     value = requests * new_tokens / dt
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     print(json.dumps({
@@ -344,6 +351,66 @@ def serving_workload(args):
     return 0
 
 
+def more_workloads(steps, warmup):
+    """What else the default line carries, each measured like the headline but shorter: the true
+    32-bit path at the Qwen3-8B sizes (decode at batch 8, a 2048-token prompt), decode at batch 8
+    at the Qwen3-32B sizes, and the reference's own benchmark shape at the Qwen3-0.6B sizes.
+    Flat: numbers, and for each workload one string that names its sizes."""
+    import gc
+
+    import torch
+
+    from litellmengine_amd.config import Qwen3Config
+    from litellmengine_amd.models import random_model
+
+    def sizes_of(cfg, what):
+        return (f"{what}: {cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, {cfg.num_attention_heads}/"
+                f"{cfg.num_key_value_heads} heads of {cfg.head_dim}, intermediate {cfg.intermediate_size}, vocab "
+                f"{cfg.vocab_size}, page {PAGE_SIZE}, random weights")
+
+    def free():
+        gc.collect()
+        torch.cuda.empty_cache()
+
+    more = {}
+    steps, warmup = max(4, min(steps, 10)), max(1, min(warmup, 2))
+    cfg = Qwen3Config.from_dict(SIZES)
+    model = random_model(cfg, seed=0, dtype="float32")
+    dt = time_decode(model, cfg, 8, 4096, steps, warmup)
+    step_bytes = weight_bytes_per_step(cfg, 4) + 8 * (4096 - (steps - 1) / 2.0) * kv_bytes_per_token(cfg, 4)
+    pt = time_prefill(model, cfg, PREFILL_TOKENS, repeats=1)
+    more.update({
+        "fp32_8b": sizes_of(cfg, "true 32-bit path, Qwen3-8B sizes, decode batch 8 at context 4096 and a 2048-token prompt"),
+        "fp32_8b_decode_b8_tok_s": round(8 / dt, 2), "fp32_8b_decode_b8_ms": round(dt * 1e3, 3),
+        "fp32_8b_decode_b8_hbm_frac": round(step_bytes / dt / HBM_PEAK, 4),
+        "fp32_8b_prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "fp32_8b_prefill_ms": round(pt * 1e3, 2),
+        "fp32_8b_prefill_frac": round(prefill_flops(cfg, PREFILL_TOKENS) / pt / MFMA_PEAK["fp32"], 4),
+    })
+    del model
+    free()
+    cfg = Qwen3Config.from_dict(SIZES_32B)
+    model = random_model(cfg, seed=0, dtype="bfloat16")
+    dt = time_decode(model, cfg, 8, 4096, steps, warmup)
+    step_bytes = weight_bytes_per_step(cfg, 2) + 8 * (4096 - (steps - 1) / 2.0) * kv_bytes_per_token(cfg, 2)
+    more.update({
+        "bf16_32b": sizes_of(cfg, "Qwen3-32B sizes, bf16, decode batch 8 at context 4096"),
+        "bf16_32b_decode_b8_tok_s": round(8 / dt, 2), "bf16_32b_decode_b8_ms": round(dt * 1e3, 3),
+        "bf16_32b_decode_b8_hbm_frac": round(step_bytes / dt / HBM_PEAK, 4),
+    })
+    del model
+    free()
+    cfg, requests, prompt_len, new_tokens, dt = time_reference_workload("bfloat16", 3, 1)
+    more.update({
+        "bf16_0p6b_reference_shape": sizes_of(cfg, f"Qwen3-0.6B sizes, bf16, {requests} requests x {prompt_len}-token prompts x "
+                                              f"{new_tokens} new tokens, prompts included (the shape of the reference's "
+                                              f"{REFERENCE_TOK_S} tok/s, which is FP32 on an unnamed CUDA GPU)"),
+        "bf16_0p6b_reference_shape_tok_s": round(requests * new_tokens / dt, 1),
+        "bf16_0p6b_reference_shape_ms": round(dt * 1e3, 2),
+    })
+    free()
+    return more
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -354,6 +421,7 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-more", action="store_true", help="skip the other workloads that the default line carries")
     ap.add_argument("--sizes", default="8b", choices=["8b", "0p6b", "32b"],
                     help="layer sizes of the decode workload: Qwen3-8B (default, the headline), Qwen3-0.6B or Qwen3-32B")
     ap.add_argument("--workload", default="decode", choices=["decode", "reference-0p6b", "mixed-32b", "serving"],
@@ -432,6 +500,11 @@ def main():
             s = max(8, args.steps // 2)
             points[f"decode_b{b}"] = round(b / time_decode(model, cfg, b, args.context, s, 4), 2)
         line["points"] = points
+        headline = (args.sizes == "8b" and args.dtype == "bfloat16" and layers == SIZES["num_hidden_layers"]
+                    and args.batch == 8 and args.context == 4096)
+        if headline and not args.no_more:
+            del model
+            line["more"] = more_workloads(args.steps, args.warmup)
     print(json.dumps(line))
     return 0
 

@@ -225,6 +225,12 @@ class HipOps:
                 slices = self.slices_for(M, N, K)
                 if slices:
                     return PartialSums(self.linear_slices(x, weight, slices))
+                slices = self.library_slices_for(M, N, K)
+                if slices:
+                    # one batched library product over the slices of K, partial sums left in 32-bit
+                    xs = x.view(M, slices, K // slices).permute(1, 0, 2)
+                    ws = weight.view(N, slices, K // slices).permute(1, 2, 0)
+                    return PartialSums(torch.bmm(xs, ws, out_dtype=torch.float32))
             skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.SKINNY_MAX_ROWS
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
@@ -287,6 +293,25 @@ class HipOps:
         return 0
 
     SLICED_LONG_K_MIN_WEIGHT = 1 << 23  # elements: below, a launch is as short as a launch can be either way
+
+    def library_slices_for(self, M: int, N: int, K: int) -> int:
+        """In how many slices of K the LIBRARY takes a product of more than 128 rows whose result is a
+        delta of the residual stream, or 0 for the whole product.  The library cuts the result into
+        tiles of up to 256 x 256 and does not split K: a weight with few rows and a long K
+        (down_proj) leaves CUs without a tile or gets small tiles.  Slices are tiles as well (one
+        batched product), up to 4 while the CUs have room for them; the residual add + norm then
+        reads float32 partial sums, which costs part of the gain.  Measured at 4096 x 12288 against
+        the whole product, both with the norm: 512 rows 90 -> 65 us (4 slices), 1024 rows 126 -> 106
+        (4), 2048 rows 214 -> 205 (2), 4096 rows slower (not taken); square weights (o_proj) gain nothing."""
+        if M <= self.SLICED_MAX_ROWS or self.force_library_gemm or K < 2 * N:
+            return 0
+        if N > MAX_SUMMED_NORM_WIDTH or N % 4 != 0:
+            return 0
+        tiles = -(-M // 256) * -(-N // 256)
+        slices = min(4, self.compute_units() // tiles)
+        while slices > 1 and K % (8 * slices) != 0:
+            slices -= 1
+        return slices if slices > 1 else 0
 
     def linear_slices(self, x, weight, slices: int) -> torch.Tensor:
         """x [M, K] . weight [N, K]^T as float32 partial sums over `slices` equal parts of K:

@@ -13,6 +13,8 @@ def load_for_generation(model_dir: str, dtype="bfloat16", device=None, random_we
     if device is not None:
         device = torch.device(device)
         if device.type == "cuda":
+            if device.index is None:  # "cuda": the current device
+                device = torch.device("cuda", torch.cuda.current_device())
             torch.cuda.set_device(device)
     if random_weights:
         return random_model(load_config(model_dir), seed, dtype, device)

@@ -311,8 +311,11 @@ def test_text_front_in_process_and_through_the_command_line(tmp_path, capsys):
     cfg, w = plain.read_model_dir(d)
     prompt = "what is the capital of france"
     start, end = tok.token_to_id("<|im_start|>"), tok.token_to_id("<|im_end|>")
-    ids = [start, 1] + [3, 4, 5, 6, 7, 8] + [end, start, 2]  # the template's line ends are no words
-    assert tok.encode("<|im_start|>user\n" + prompt + "<|im_end|>\n<|im_start|>assistant\n", add_special_tokens=False).ids == ids
+    from litellmengine_amd.entrypoints.cli import templated_prompt
+
+    # the architecture's template around the prompt (thinking off: an empty block of thoughts, unknown words here)
+    ids = tok.encode(templated_prompt(d, prompt, enable_thinking=False), add_special_tokens=False).ids
+    assert ids[:11] == [start, 1] + [3, 4, 5, 6, 7, 8] + [end, start, 2] and len(ids) > 11
     want = plain.generate_greedy(ids, w, cfg, 6, eos=end)
     text = tok.decode(want, skip_special_tokens=True)
     common = ["--model", d, "--prompt", prompt, "--max-tokens", "6", "--dtype", "float32", "--show-full-text"]

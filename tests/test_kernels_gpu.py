@@ -224,6 +224,25 @@ def test_which_products_are_taken_in_slices():
         # no whole rounds; a square weight in a round and a quarter (o_proj of the 32B sizes) stays the library's
         assert o.slices_for(64, 5120, 25600) == 5 and o.slices_for(64, 5120, 17408) == 17
         assert o.slices_for(64, 5120, 8192) == 0 and o.slices_for(64, 1024, 3072) == 0
+    if units == 256:
+        # the library's products (more than 128 rows) of a weight with few rows and a long K: slices while the
+        # CUs have room for the tiles; not for square weights, not when the tiles fill the CUs anyway
+        assert [o.library_slices_for(m, 4096, 12288) for m in (128, 129, 512, 1024, 2048, 4096)] == [0, 4, 4, 4, 2, 0]
+        assert o.library_slices_for(2048, 4096, 4096) == 0 and o.library_slices_for(1024, 5120, 25600) == 2
+        assert o.library_slices_for(512, 8192 + 256, 32768) == 0  # wider than the norm that adds the slices up takes
+    x = rnd((300, 12288), torch.bfloat16, 67, 0.5)
+    w = rnd((1024, 12288), torch.bfloat16, 68, 0.05)
+    got = o.linear(x, w, sums_ok=True)
+    assert got.sums.shape == (4, 300, 1024) and got.sums.dtype == torch.float32
+    want = x.double() @ w.double().t()
+    assert (got.total().double() - want).abs().max() < 1e-3 * want.abs().max()  # float32 sums of bfloat16 products
+    hidden = rnd((300, 1024), torch.float32, 69)
+    nw = (1 + 0.1 * rnd((1024,), torch.float32, 70)).bfloat16()
+    h_want = hidden.double() + want
+    normed = o.add_rmsnorm(hidden, got, nw, 1e-6, torch.bfloat16)
+    assert (hidden.double() - h_want).abs().max() < 1e-3 * want.abs().max()
+    n_want = h_want / torch.sqrt((h_want * h_want).mean(-1, keepdim=True) + 1e-6) * nw.double()
+    assert (normed.double() - n_want).abs().max() < 3e-2
     x = rnd((40, 4096), torch.bfloat16, 65)
     w = rnd((n, 4096), torch.bfloat16, 66, 0.05)
     assert o.linear(x, w).shape == (40, n)                       # a caller that said nothing gets the product

@@ -447,7 +447,7 @@ def test_a_mixer_with_state_decodes_through_graphs(dtype):
         assert cache.states[0].shape == (3 + 1, hidden + 1)  # a spare row for the rows that pad a batch
         runner = ModelRunner(model, cache, use_graphs=use_graphs)
         assert runner.use_graphs == use_graphs
-        seqs = [random_tokens(30, vocab, 11), random_tokens(22, vocab, 12)]
+        seqs = [random_tokens(30, vocab, 11), random_tokens(18, vocab, 12)]
         slots = [runner.admit(), runner.admit()]
         got = [[], []]
         got[0].append(runner.step([StepEntry(slots[0], seqs[0][:9], list(range(9)))]))
