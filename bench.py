@@ -311,7 +311,7 @@ def serving_workload(args):
     engine = LLMEngine(model, page_size=PAGE_SIZE, num_pages=pages_each * live, max_requests=live,
                        max_tokens_per_step=PREFILL_TOKENS, max_pages_per_request=pages_each)
     todo = [(random_prompts(1, p, cfg.vocab_size, 100 + i)[0], g) for i, (p, g) in enumerate(sizes)]
-    kinds = collections.defaultdict(lambda: [0, 0.0])
+    kinds = collections.defaultdict(lambda: [0, 0.0])  # kind -> steps, seconds, then the tokens of every such step
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     steps = 0
@@ -320,16 +320,18 @@ def serving_workload(args):
             prompt, new = todo.pop(0)
             engine.add_request(prompt, new)
         before = sum(r.cached_len for r in engine.scheduler.requests.values())
-        captures = engine.runner.num_captures
+        captures, graph_steps = engine.runner.num_captures, engine.runner.num_graph_steps
         ts = time.perf_counter()
         engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - ts
         ran = sum(r.cached_len for r in engine.scheduler.requests.values()) - before
         kind = ("capture" if engine.runner.num_captures > captures else
+                "decode_only_graph" if engine.runner.num_graph_steps > graph_steps else
                 "le64" if ran <= 64 else "le256" if ran <= 256 else "le1024" if ran <= 1024 else "gt1024")
         kinds[kind][0] += 1
         kinds[kind][1] += dt
+        kinds[kind].append(ran)
         steps += 1
     total = time.perf_counter() - t0
     new_tokens = sum(g for _, g in sizes)
@@ -345,8 +347,9 @@ def serving_workload(args):
                               global_batch=live, requests=requests, token_budget=PREFILL_TOKENS),
         "new_tokens_per_s": round(new_tokens / total, 1), "seconds": round(total, 3),
         "graph_captures": engine.runner.num_captures,
-        "steps_by_tokens": {k: {"steps": n, "ms_each": round(t / n * 1e3, 2), "share": round(t / total, 3)}
-                            for k, (n, t) in sorted(kinds.items())},
+        "steps_by_tokens": {k: {"steps": v[0], "ms_each": round(v[1] / v[0] * 1e3, 2), "share": round(v[1] / total, 3),
+                                "tokens_each": round(sum(v[2:]) / v[0], 1)}
+                            for k, v in sorted(kinds.items())},
     }))
     return 0
 

@@ -279,6 +279,14 @@ class CacheManager:
         self._check_live(slot)
         return self._length[slot]
 
+    def lengths_of(self, slots: Sequence[int]) -> List[int]:
+        """length() of every slot in `slots` (all must be in use)."""
+        live, length, most = self._live, self._length, self.max_requests
+        for slot in slots:
+            if not (0 <= slot < most and live[slot]):
+                raise ValueError(f"request slot {slot} is not in use")
+        return [length[slot] for slot in slots]
+
     def _check_live(self, slot: int) -> None:
         if not self.is_live(slot):
             raise ValueError(f"request slot {slot} is not in use")

@@ -1,4 +1,4 @@
-// Embedding row gather and SiLU-and-mul.
+// Embedding row gather, SiLU-and-mul and the bias of a projection.
 // Counterparts in the reference: embedding_forward_kernel
 // (src/layers/embedding.cu:91-118) and silu_and_mul_kernel
 // (src/ops/silu_and_mul.cu:64-80); both are 32-bit only there.
@@ -78,5 +78,29 @@ extern "C" int lle_silu_mul(const void* gate_up, void* out, int N, int I, int dt
         silu_mul_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, total, I);
     else
         silu_mul_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, total, I);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
+// x[m, :] += bias[:] in place, the sum in 32-bit (the reference's Linear has the same optional
+// bias, src/layers/linear.cu:169-215; Qwen3 uses none).  `bias` holds TB, x holds T.
+template <typename T, typename TB>
+__global__ __launch_bounds__(256) void add_bias_kernel(T* __restrict__ x, const TB* __restrict__ bias, int64_t total,
+                                                        int N) {
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (int64_t)gridDim.x * blockDim.x)
+        x[idx] = from_f32<T>(to_f32<T>(x[idx]) + to_f32<TB>(bias[idx % N]));
+}
+
+extern "C" int lle_add_bias(void* x, const void* bias, int M, int N, int dtype, int bias_dtype, hipStream_t stream) {
+    const int64_t total = (int64_t)M * N;
+    if (total <= 0) return 0;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+#define LLE_BIAS_CASE(T, TB) add_bias_kernel<T, TB><<<(int)blocks, 256, 0, stream>>>((T*)x, (const TB*)bias, total, N)
+    if (dtype == LLE_F32 && bias_dtype == LLE_F32) LLE_BIAS_CASE(float, float);
+    else if (dtype == LLE_F32) LLE_BIAS_CASE(float, bf16_t);
+    else if (bias_dtype == LLE_F32) LLE_BIAS_CASE(bf16_t, float);
+    else LLE_BIAS_CASE(bf16_t, bf16_t);
+#undef LLE_BIAS_CASE
     LLE_RETURN_LAUNCH_STATUS();
 }

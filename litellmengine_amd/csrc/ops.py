@@ -605,6 +605,15 @@ class HipOps:
         by_fill = max(1, self.compute_units() // max(1, num_seqs * num_kv_heads))
         return int(min(by_work, by_fill, 64))
 
+    def add_bias(self, x, bias) -> torch.Tensor:
+        """x [M, N] += bias [N], in place (the sum in 32-bit); returns x."""
+        _dev(x, "x")
+        _dev(bias, "bias")
+        _need(x.dim() == 2 and bias.shape == (x.shape[1],), f"bias {list(bias.shape)} does not fit x {list(x.shape)}")
+        self._run("elementwise", "lle_add_bias", [_P, _P, _I, _I, _I, _I, _P], _ptr(x), _ptr(bias), x.shape[0],
+                  x.shape[1], dtype_code(x.dtype), dtype_code(bias.dtype))
+        return x
+
     # -- feed-forward --------------------------------------------------------------
     def silu_mul(self, gate_up) -> torch.Tensor:
         """gate_up [N, 2 I] (gate columns first) -> silu(gate) * up, [N, I]."""

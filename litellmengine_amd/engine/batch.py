@@ -12,15 +12,14 @@ from __future__ import annotations
 import ctypes
 import dataclasses
 from array import array
-from typing import List, Optional, Sequence, Tuple
+from typing import List, NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
 from ..cache.page_pool import BAD_TOKEN, NO_PAGE_AT_POSITION, host_library
 
 
-@dataclasses.dataclass(frozen=True)
-class StepEntry:
+class StepEntry(NamedTuple):
     """A request's share of a step: its cache slot, its next tokens and the
     places among them (0-based) whose logits are wanted."""
 
@@ -29,8 +28,7 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
-@dataclasses.dataclass(frozen=True)
-class SeqInfo:
+class SeqInfo(NamedTuple):
     slot: int
     q_start: int  # first row of the request in the flat batch
     q_len: int
@@ -64,8 +62,9 @@ class StepLayout:
     num_seqs: int
     num_logit_rows: int
     num_groups: int
-    seqs: List[SeqInfo]
+    seqs: Optional[List[SeqInfo]]  # None when the caller asked for none
     max_kv_len: int
+    q_lens: Tuple[int, int] = (1, 1)  # fewest and most tokens of a request in this step
 
     def sizes(self) -> List[int]:
         N, S, R = self.num_tokens, self.num_seqs, self.num_logit_rows
@@ -93,35 +92,48 @@ _staging = _Staging()
 
 
 def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, vocab_size: int = 0,
-                device=None, pad_to: int = 0) -> StepLayout:
+                device=None, pad_to: int = 0, with_seqs: bool = True) -> StepLayout:
     """Lay the entries out flat and compute every token's page slot in every cache
     group (csrc/host.cpp does both).  Pages for the new lengths must already be there.
     `all_rows` asks for the logits of every row whatever the entries want; with
     `vocab_size` token ids outside [0, vocab_size) are refused.  `pad_to` fills the batch
     up to that many requests with single tokens that stand for nobody: they read the
-    cache's spare table row and page (`cache.pad_slot`) and write nothing."""
+    cache's spare table row and page (`cache.pad_slot`) and write nothing.  Without
+    `with_seqs` the host-side list of the requests is left out (a step that runs as a graph
+    has no use for it, and it costs as much as everything else here)."""
     S = len(entries)
     pad = max(0, pad_to - S)
-    slots = array("i", (e.slot for e in entries))
-    past = array("i", (cache.length(e.slot) for e in entries))
-    q_len = array("i", (len(e.tokens) for e in entries))
+    slots = array("i", [e.slot for e in entries])
+    lengths = cache.lengths_of(slots)
+    past = array("i", lengths)
+    q_len = array("i", [len(e.tokens) for e in entries])
     tokens = array("i")
     rows = array("i")
-    seqs: List[SeqInfo] = []
+    seqs: Optional[List[SeqInfo]] = [] if with_seqs else None
     start = 0
-    for e, p, n in zip(entries, past, q_len):
-        tokens.extend(e.tokens if isinstance(e.tokens, (list, array)) else [int(t) for t in e.tokens])
-        if all_rows:
-            rows.extend(range(start, start + n))
-        else:
-            rows.extend(start + int(w) for w in e.want)
-        seqs.append(SeqInfo(e.slot, start, n, p))
-        start += n
+    if all_rows and max(q_len, default=1) == 1:  # single tokens: row i is request i's
+        for e in entries:
+            tokens.extend(e.tokens if isinstance(e.tokens, (list, array)) else [int(t) for t in e.tokens])
+        start = S
+        rows.extend(range(S))
+        if with_seqs:
+            seqs.extend(SeqInfo(e.slot, i, 1, p) for i, (e, p) in enumerate(zip(entries, past)))
+    else:
+        for e, p, n in zip(entries, past, q_len):
+            tokens.extend(e.tokens if isinstance(e.tokens, (list, array)) else [int(t) for t in e.tokens])
+            if all_rows:
+                rows.extend(range(start, start + n))
+            else:
+                rows.extend(start + int(w) for w in e.want)
+            if with_seqs:
+                seqs.append(SeqInfo(e.slot, start, n, p))
+            start += n
     N, G = start, len(cache.groups)
     if pad:
         if all_rows:
             rows.extend(range(N, N + pad))
-        seqs.extend(SeqInfo(cache.pad_slot, N + i, 1, 0) for i in range(pad))
+        if with_seqs:
+            seqs.extend(SeqInfo(cache.pad_slot, N + i, 1, 0) for i in range(pad))
     R = len(rows)
     pinned = device is not None and torch.device(device).type == "cuda"
     host = _staging.get(3 * (N + pad) + 3 * (S + pad) + 1 + R + G * (N + pad), pinned)
@@ -138,7 +150,8 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
         raise IndexError(f"position {info.value} has no page: the cache was not extended for this step")
     if code != 0:
         raise ValueError(f"the step cannot be laid out: {lib.lle_error_string(code).decode()} (at {info.value})")
-    return StepLayout(host, N + pad, S + pad, R, G, seqs, max((p + n for p, n in zip(past, q_len)), default=1))
+    q_lens = (min(q_len, default=1) if not pad else 1, max(q_len, default=1))
+    return StepLayout(host, N + pad, S + pad, R, G, seqs, max((p + n for p, n in zip(past, q_len)), default=1), q_lens)
 
 
 def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:
@@ -176,7 +189,7 @@ def state_on(buf: torch.Tensor, layout: StepLayout, cache, max_kv_len: Optional[
     return StepState(
         num_tokens=layout.num_tokens, num_seqs=layout.num_seqs, token_ids=v[0], positions=v[1], token_seq=v[2],
         seq_slots=v[3], cu_tokens=v[4], kv_lens=v[5], logit_rows=v[6],
-        min_q_len=min(q.q_len for q in layout.seqs), max_q_len=max(q.q_len for q in layout.seqs),
+        min_q_len=layout.q_lens[0], max_q_len=layout.q_lens[1],
         max_kv_len=max_kv_len or layout.max_kv_len, seqs=layout.seqs if with_seqs else None,
     )
 

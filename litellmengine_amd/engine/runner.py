@@ -57,6 +57,7 @@ class ModelRunner:
         self._graphs: "collections.OrderedDict[Tuple[int, int], _DecodeGraph]" = collections.OrderedDict()
         self._graph_pool = None
         self.num_captures = 0
+        self.num_graph_steps = 0  # steps that ran as a graph (decode steps), captures included
         if self.use_graphs:
             self._first_graph_of_the_process(self.device)
 
@@ -94,18 +95,18 @@ class ModelRunner:
     def check(self, entries: Sequence[StepEntry]) -> None:
         if not entries:
             raise ValueError("a step needs at least one entry")
-        seen = set()
+        slots = [e.slot for e in entries]
+        if len(set(slots)) != len(slots):
+            twice = next(s for i, s in enumerate(slots) if s in slots[:i])
+            raise ValueError(f"request slot {twice} appears twice in one step")
+        self.cache.lengths_of(slots)  # (every slot is in use)
         for e in entries:
-            if e.slot in seen:
-                raise ValueError(f"request slot {e.slot} appears twice in one step")
-            seen.add(e.slot)
-            if not self.cache.is_live(e.slot):
-                raise ValueError(f"request slot {e.slot} is not in use")
-            if len(e.tokens) == 0:
+            n = len(e.tokens)
+            if n == 0:
                 raise ValueError("an entry needs at least one token")
             for w in e.want:
-                if not 0 <= int(w) < len(e.tokens):
-                    raise ValueError(f"wanted place {w} outside the entry's {len(e.tokens)} tokens")
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"wanted place {w} outside the entry's {n} tokens")
 
     def check_tokens(self, entries: Sequence[StepEntry]) -> None:
         """Token ids outside the vocabulary are refused before anything is changed
@@ -145,9 +146,10 @@ class ModelRunner:
     # decoding through a captured graph ---------------------------------------------------
     def _graph_step(self, entries: Sequence[StepEntry], borrow: bool) -> torch.Tensor:
         cache = self.cache
+        self.num_graph_steps += 1
         batch = next(b for b in self.BATCH_BUCKETS if b >= len(entries))
         layout = layout_step(entries, cache, all_rows=True, vocab_size=self.vocab_size, device=self.device,
-                             pad_to=batch)
+                             pad_to=batch, with_seqs=False)
         apply_table_updates(cache, self.device)
         bucket = self.MIN_CONTEXT_BUCKET
         while bucket < layout.max_kv_len:
@@ -181,7 +183,7 @@ class ModelRunner:
         # every mixer's state, nothing written.  So no request's cache or state moves before the
         # graph's first replay, whatever the mixers keep.
         warm = layout_step([], self.cache, all_rows=True, vocab_size=self.vocab_size, device=self.device,
-                           pad_to=layout.num_seqs)
+                           pad_to=layout.num_seqs, with_seqs=False)
         warm_state = state_on(warm.host.to(self.device), warm, self.cache, max_kv_len=bucket, with_seqs=False)
         side = torch.cuda.Stream(device=self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))

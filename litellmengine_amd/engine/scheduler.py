@@ -34,15 +34,13 @@ are too few, nothing is evicted and the request goes on waiting.
 from __future__ import annotations
 
 import collections
-import dataclasses
-from typing import Deque, Dict, List, Optional, Sequence
+from typing import Deque, Dict, List, NamedTuple, Optional, Sequence
 
 from ..cache import CacheManager, OutOfPages
 from .request import Request, RequestStatus
 
 
-@dataclasses.dataclass(frozen=True)
-class Portion:
+class Portion(NamedTuple):
     """`num_tokens` tokens of `request` from its `cached_len` on; `samples` when
     the portion reaches the end of what the request has, so a token is drawn."""
 

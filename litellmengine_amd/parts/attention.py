@@ -14,7 +14,7 @@ reference has full attention only).
 from __future__ import annotations
 
 import math
-from typing import Dict, Optional
+from typing import Dict, Optional, Sequence
 
 import torch
 
@@ -39,7 +39,17 @@ class PagedAttention(Mixer):
         qk_norm_eps: Optional[float] = None,
         window: Optional[int] = None,
         scale: Optional[float] = None,
+        qkv_names: Optional[Sequence[str]] = None,
+        o_name: Optional[str] = None,
+        qkv_bias: bool = False,
+        o_bias: bool = False,
+        qk_norm_names: Optional[Sequence[str]] = None,
     ):
+        """`qkv_names`: the checkpoint's names of the projections' weights after `prefix`, three
+        (q, k, v; default q_proj.weight, k_proj.weight, v_proj.weight) or one that holds the three
+        stacked in that order; `o_name` the output projection's (default o_proj.weight);
+        `qk_norm_names` the two norm weights' (default q_norm.weight, k_norm.weight).  With
+        `qkv_bias` / `o_bias` every weight `x.weight` has a bias `x.bias`."""
         if num_q_heads % num_kv_heads:
             raise ValueError("num_q_heads must be a multiple of num_kv_heads")
         check_head_dim(head_dim, getattr(position, "rotary_dim", 0))  # what no kernel takes is refused now, not at the first step
@@ -49,12 +59,22 @@ class PagedAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps
         self.window = window
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else float(scale)
-        self.qkv = Linear(
-            [prefix + "q_proj.weight", prefix + "k_proj.weight", prefix + "v_proj.weight"],
-            hidden_size,
-            [num_q_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim],
-        )
-        self.o = Linear([prefix + "o_proj.weight"], num_q_heads * head_dim, [hidden_size], to_residual=True)
+        widths = [num_q_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * head_dim]
+        names = list(qkv_names) if qkv_names else ["q_proj.weight", "k_proj.weight", "v_proj.weight"]
+        if len(names) == 1:
+            widths = [sum(widths)]  # the three stacked in one checkpoint tensor
+        elif len(names) != 3:
+            raise ValueError("qkv_names holds three names (q, k, v) or one (the three stacked)")
+        o_name = o_name or "o_proj.weight"
+        bias_of = lambda name: prefix + (name[: -len("weight")] + "bias" if name.endswith("weight") else name + ".bias")
+        self.qkv = Linear([prefix + n for n in names], hidden_size, widths,
+                          bias_names=[bias_of(n) for n in names] if qkv_bias else None)
+        self.o = Linear([prefix + o_name], num_q_heads * head_dim, [hidden_size], to_residual=True,
+                        bias_names=[bias_of(o_name)] if o_bias else None)
+        self.folds_norm = not o_bias  # (the product before a folded norm adds into the residual stream itself)
+        self.qk_norm_names = list(qk_norm_names) if qk_norm_names else ["q_norm.weight", "k_norm.weight"]
+        if len(self.qk_norm_names) != 2:
+            raise ValueError("qk_norm_names holds two names (q, k)")
         self.q_norm_w = None
         self.k_norm_w = None
 
@@ -64,8 +84,8 @@ class PagedAttention(Mixer):
     def tensor_specs(self) -> Dict[str, TensorSpec]:
         specs = {**self.qkv.tensor_specs(), **self.o.tensor_specs()}
         if self.qk_norm_eps is not None:
-            specs[self.prefix + "q_norm.weight"] = TensorSpec((self.d,), INIT_NORM)
-            specs[self.prefix + "k_norm.weight"] = TensorSpec((self.d,), INIT_NORM)
+            for name in self.qk_norm_names:
+                specs[self.prefix + name] = TensorSpec((self.d,), INIT_NORM)
         return specs
 
     def bind(self, weights, ctx: BuildContext) -> None:
@@ -74,8 +94,8 @@ class PagedAttention(Mixer):
         self.o.bind(weights, ctx)
         self.position.bind(weights, ctx)
         if self.qk_norm_eps is not None:
-            qw = weights[self.prefix + "q_norm.weight"]
-            kw = weights[self.prefix + "k_norm.weight"]
+            qw = weights[self.prefix + self.qk_norm_names[0]]
+            kw = weights[self.prefix + self.qk_norm_names[1]]
             if qw.dtype != kw.dtype:
                 qw, kw = qw.float(), kw.float()
             self.q_norm_w, self.k_norm_w = qw.contiguous(), kw.contiguous()

@@ -479,3 +479,46 @@ def test_a_mixer_with_state_decodes_through_graphs(dtype):
         for use_graphs in (True, False):
             err = (outs[use_graphs][i] - want).abs().max().item()
             assert err < TOL[dtype], (i, use_graphs, err)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("packed", [False, True], ids=["three tensors", "one stacked tensor"])
+def test_attention_with_biases_and_other_tensor_names(dtype, packed):
+    """The attention mixer with what another architecture's checkpoint may bring: a bias on
+    the q/k/v and on the output projection, the three projections stacked in one tensor, norm
+    weights under other names.  Parameters of the part, no change to it; stepped in portions
+    and single tokens (small steps: the products beside a folded norm run too) against the plain formulas."""
+    H, nq, nkv, d, I, T = 64, 4, 2, 32, 96, 17
+    p = "blk.attn."
+    names = ["Wqkv.weight"] if packed else ["query.weight", "key.weight", "value.weight"]
+    mixer = PagedAttention(p, H, nq, nkv, d, RotaryHalfSplit(d, 1e4), qk_norm_eps=1e-5, qkv_names=names, o_name="dense.weight",
+                           qkv_bias=True, o_bias=True, qk_norm_names=["ln_q.weight", "ln_k.weight"])
+    assert not mixer.folds_norm and mixer.qkv.has_bias and mixer.o.has_bias
+    expected = {p + n for n in names} | {p + n[:-6] + "bias" for n in names}
+    expected |= {p + "dense.weight", p + "dense.bias", p + "ln_q.weight", p + "ln_k.weight"}
+    assert set(mixer.tensor_specs()) == expected
+    block = PreNormBlock(RMSNorm("blk.n1", H, 1e-5), mixer, RMSNorm("blk.n2", H, 1e-5), GatedMLP("blk.mlp.", H, I))
+    model = one_block_model(block, H)
+    ctx, w = bound(model, dtype, seed=3)
+    model.ctx = ctx
+    cache = CacheManager(model, page_size=16, num_pages=4, max_requests=2, dtype=dtype, device=ctx.device)
+    runner = ModelRunner(model, cache)
+    ids = random_tokens(T, 50, 8)
+    x0 = plain.embedding(ids, w["e.weight"])
+    xn = plain.rms_norm(x0, w["blk.n1"], 1e-5)
+    if packed:
+        qkv = plain.linear(xn, w[p + "Wqkv.weight"]) + w[p + "Wqkv.bias"]
+        q, k, v = qkv[:, : nq * d], qkv[:, nq * d : (nq + nkv) * d], qkv[:, (nq + nkv) * d :]
+    else:
+        q, k, v = (plain.linear(xn, w[p + n + ".weight"]) + w[p + n + ".bias"] for n in ("query", "key", "value"))
+    q = plain.rope_half_split(plain.rms_norm(q.reshape(T, nq, d), w[p + "ln_q.weight"], 1e-5), range(T), 1e4)
+    k = plain.rope_half_split(plain.rms_norm(k.reshape(T, nkv, d), w[p + "ln_k.weight"], 1e-5), range(T), 1e4)
+    a = plain.causal_gqa_attention(q, k, v.reshape(T, nkv, d)).reshape(T, nq * d)
+    r = x0 + plain.linear(a, w[p + "dense.weight"]) + w[p + "dense.bias"]
+    r = r + plain.gated_mlp(plain.rms_norm(r, w["blk.n2"], 1e-5), w["blk.mlp.gate_proj.weight"],
+                            w["blk.mlp.up_proj.weight"], w["blk.mlp.down_proj.weight"])
+    want = plain.fast_linear(plain.rms_norm(r, w["fn.weight"], 1e-6), w["head.weight"])
+    slot = runner.admit()
+    got = torch.cat([runner.step([StepEntry(slot, ids[a0:b0], list(range(b0 - a0)))]).cpu()
+                     for a0, b0 in ((0, 9), (9, 10), (10, 11), (11, 17))])
+    assert (got.double() - want).abs().max() < TOL[dtype]

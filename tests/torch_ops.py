@@ -62,6 +62,10 @@ class TorchOps:
         assert fold is None, "this stand-in folds no norm (can_fold_norm says so)"
         return (x.to(self.cd) @ weight.to(self.cd).t()).to(out_dtype or x.dtype)
 
+    def add_bias(self, x, bias):
+        x += bias.to(x.dtype)
+        return x
+
     def rope_table(self, positions, inv_freq):
         ang = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).double()  # float32 product
         return torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).to(torch.float32)
