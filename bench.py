@@ -140,17 +140,19 @@ def measure_peaks(dtype):
 
     ops = default_ops()
 
-    def timed(launch):
+    def timed(launch, repeats=8):
+        # by the wall clock around a run of launches (no timing events: recording one makes the runtime
+        # keep time stamps of every later launch of the process, which costs the short kernels of a
+        # decode step about a microsecond each)
         launch()
         torch.cuda.synchronize()
         best = None
         for _ in range(3):
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record()
-            launch()
-            end.record()
-            end.synchronize()
-            dt = start.elapsed_time(end) * 1e-3
+            t0 = time.perf_counter()
+            for _ in range(repeats):
+                launch()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / repeats
             best = dt if best is None else min(best, dt)
         return best
 
@@ -167,7 +169,7 @@ def measure_peaks(dtype):
     def mfma():
         flops[0] = ops.probe_mfma(tdtype, 8 * units, 4000)
 
-    seconds = timed(mfma)
+    seconds = timed(mfma, repeats=2)
     return read, flops[0] / seconds
 
 

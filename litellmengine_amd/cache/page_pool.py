@@ -40,7 +40,7 @@ _SIGNATURES = {
     "lle_pt_token_slot": ([_P, _I, _I], _L),
     "lle_pt_num_pending": ([_P], _I),
     "lle_pt_take_pending": ([_P, _P, _P], None),
-    "lle_layout_step": ([_I, _P, _P, _P, _P, _I, _I, _P, _I, _P, _I, _I, _P, _P], _I),
+    "lle_layout_step": ([_I, _P, _P, _P, _P, _I, _I, _I, _P, _I, _P, _I, _I, _P, _P], _I),
 }
 _lib = None
 

@@ -8,24 +8,46 @@ LLE_DEFINE_ERROR_STRING()
 
 // out[n, :] = table[ids[n], :] as 32-bit (the residual stream is 32-bit in
 // every mode).  The host has checked 0 <= id < V.
+// An id below zero stands for "the token that the last step picked for this token's request": it
+// is read from feedback[seq_slots[token_seq[n]]], where the picking kernel left it (a step that
+// was launched before the host had read the step before it; the picking kernel only writes ids
+// of the vocabulary).
 template <typename T>
 __global__ __launch_bounds__(256) void embedding_kernel(const int32_t* __restrict__ ids,
                                                          const T* __restrict__ table,
-                                                         float* __restrict__ out, int H) {
+                                                         float* __restrict__ out, int H,
+                                                         const int32_t* __restrict__ feedback,
+                                                         const int32_t* __restrict__ token_seq,
+                                                         const int32_t* __restrict__ seq_slots) {
     const int64_t n = blockIdx.x;
-    const T* row = table + (int64_t)ids[n] * H;
+    int id = ids[n];
+    if (id < 0) id = feedback ? feedback[seq_slots[token_seq[n]]] : 0;
+    const T* row = table + (int64_t)id * H;
     float* o = out + n * H;
     for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32<T>(row[i]);
 }
 
+// `feedback`, `token_seq` [N] and `seq_slots`: all three or none
+extern "C" int lle_embedding_feedback(const void* ids, const void* table, void* out, int N, int H, int dtype,
+                                      const void* feedback, const void* token_seq, const void* seq_slots,
+                                      hipStream_t stream) {
+    if (N <= 0) return 0;
+    if ((feedback != nullptr) != (token_seq != nullptr) || (feedback != nullptr) != (seq_slots != nullptr))
+        return (int)hipErrorInvalidValue;
+    if (dtype == LLE_F32)
+        embedding_kernel<float><<<N, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, H,
+                                                        (const int32_t*)feedback, (const int32_t*)token_seq,
+                                                        (const int32_t*)seq_slots);
+    else
+        embedding_kernel<bf16_t><<<N, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, H,
+                                                         (const int32_t*)feedback, (const int32_t*)token_seq,
+                                                         (const int32_t*)seq_slots);
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
 extern "C" int lle_embedding(const void* ids, const void* table, void* out, int N, int H, int dtype,
                              hipStream_t stream) {
-    if (N <= 0) return 0;
-    if (dtype == LLE_F32)
-        embedding_kernel<float><<<N, 256, 0, stream>>>((const int32_t*)ids, (const float*)table, (float*)out, H);
-    else
-        embedding_kernel<bf16_t><<<N, 256, 0, stream>>>((const int32_t*)ids, (const bf16_t*)table, (float*)out, H);
-    LLE_RETURN_LAUNCH_STATUS();
+    return lle_embedding_feedback(ids, table, out, N, H, dtype, nullptr, nullptr, nullptr, stream);
 }
 
 // gate_up [N, 2I] (gate columns first) -> out [N, I] = gate / (1 + exp(-gate)) * up, in 32-bit

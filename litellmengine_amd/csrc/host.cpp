@@ -268,8 +268,8 @@ void lle_pt_take_pending(void* h, int32_t* index, int32_t* pages) {
 // (a row that points at a page nobody writes), page slot -1 (nothing is written).  The sizes above
 // then count them: N + pad tokens, S + pad requests; `logit_rows` may name their rows.
 int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int32_t* q_len, const int32_t* tokens,
-                    int vocab_size, int R, const int32_t* logit_rows, int G, void* const* groups, int pad,
-                    int pad_slot, int32_t* out, int64_t* info) {
+                    int vocab_size, int allow_deferred, int R, const int32_t* logit_rows, int G, void* const* groups,
+                    int pad, int pad_slot, int32_t* out, int64_t* info) {
     // (no request at all is allowed when the batch is padding only: the warm-up of a graph's kernels)
     if (S < 0 || (S == 0 && pad <= 0) || R < 0 || G < 0 || pad < 0 || (pad > 0 && pad_slot < 0)) return LLE_HOST_BAD_ARGUMENT;
     int64_t N = 0;
@@ -280,8 +280,10 @@ int lle_layout_step(int S, const int32_t* slots, const int32_t* past, const int3
         }
         N += q_len[s];
     }
+    // (with `allow_deferred` an id of -1 stands for a token that is still on the device: the one the
+    // step before picked for this request)
     for (int64_t i = 0; i < N; ++i)
-        if (tokens[i] < 0 || (vocab_size > 0 && tokens[i] >= vocab_size)) {
+        if ((tokens[i] < 0 && !(allow_deferred && tokens[i] == -1)) || (vocab_size > 0 && tokens[i] >= vocab_size)) {
             *info = i;
             return LLE_HOST_BAD_TOKEN;
         }

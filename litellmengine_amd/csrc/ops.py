@@ -95,15 +95,24 @@ class HipOps:
             raise KernelError(f"{name} failed to launch: {msg} (hip error {code})")
 
     # -- embedding -----------------------------------------------------------
-    def embedding(self, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-        """ids int32 [N], table [V, H] -> float32 [N, H] (the residual stream)."""
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, feedback=None, token_seq=None,
+                  seq_slots=None) -> torch.Tensor:
+        """ids int32 [N], table [V, H] -> float32 [N, H] (the residual stream).  With `feedback`
+        (int32, indexed by request slot), `token_seq` [N] and `seq_slots`: an id below zero is
+        replaced by feedback[seq_slots[token_seq[n]]], the token that argmax(..., scatter=...) left there."""
         _dev(ids, "ids", torch.int32)
         _dev(table, "embedding table")
         _need(ids.dim() == 1 and table.dim() == 2, "embedding wants ids [N] and a table [V, H]")
         N, H = ids.shape[0], table.shape[1]
+        if feedback is not None:
+            for t, name in ((feedback, "feedback"), (token_seq, "token_seq"), (seq_slots, "seq_slots")):
+                _need(t is not None, "feedback, token_seq and seq_slots come together")
+                _dev(t, name, torch.int32)
+            _need(token_seq.shape == (N,), "token_seq must be [N]")
         out = torch.empty((N, H), dtype=torch.float32, device=table.device)
-        self._run("elementwise", "lle_embedding", [_P, _P, _P, _I, _I, _I, _P],
-                  _ptr(ids), _ptr(table), _ptr(out), N, H, dtype_code(table.dtype))
+        self._run("elementwise", "lle_embedding_feedback", [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P],
+                  _ptr(ids), _ptr(table), _ptr(out), N, H, dtype_code(table.dtype), _ptr(feedback),
+                  _ptr(token_seq) if feedback is not None else None, _ptr(seq_slots) if feedback is not None else None)
         return out
 
     # -- norms ---------------------------------------------------------------
@@ -645,16 +654,23 @@ class HipOps:
         return self.silu_mul(self.linear(x, weight))
 
     # -- picking tokens --------------------------------------------------------------
-    def argmax(self, logits) -> torch.Tensor:
-        """float32 [R, V] -> int32 [R], first maximum wins."""
+    def argmax(self, logits, scatter=None) -> torch.Tensor:
+        """float32 [R, V] -> int32 [R], first maximum wins.  `scatter` = (dst int32, index int32 [R]):
+        the pick of row r is also written to dst[index[r]] (the host has made sure that index is in range)."""
         _dev(logits, "logits", torch.float32)
         R, V = logits.shape
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
         chunks = max(1, min(64, V // 2048))  # enough workgroups to stream a long row from all CUs
         part_val = torch.empty((R * chunks,), dtype=torch.float32, device=logits.device)
         part_idx = torch.empty((R * chunks,), dtype=torch.int32, device=logits.device)
-        self._run("sampling", "lle_argmax_rows", [_P, _P, _P, _P, _I, _I, _I, _P],
-                  _ptr(logits), _ptr(out), _ptr(part_val), _ptr(part_idx), R, V, chunks)
+        dst = index = None
+        if scatter is not None:
+            dst, index = scatter
+            _dev(dst, "scatter destination", torch.int32)
+            _dev(index, "scatter index", torch.int32)
+            _need(index.shape == (R,), "one scatter index for every row")
+        self._run("sampling", "lle_argmax_rows_scatter", [_P, _P, _P, _P, _I, _I, _I, _P, _P, _P],
+                  _ptr(logits), _ptr(out), _ptr(part_val), _ptr(part_idx), R, V, chunks, _ptr(dst), _ptr(index))
         return out
 
     def sample(self, logits, temperature, uniform) -> torch.Tensor:

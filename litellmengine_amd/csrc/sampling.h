@@ -10,6 +10,11 @@ extern "C" {
 int lle_argmax_rows(const void* logits, void* out, void* part_val, void* part_idx, int R, int V, int chunks,
                     hipStream_t stream);
 
+// The same, and the pick of row r is also written to scatter_dst[scatter_index[r]] (both int32,
+// both given or neither).
+int lle_argmax_rows_scatter(const void* logits, void* out, void* part_val, void* part_idx, int R, int V, int chunks,
+                            void* scatter_dst, const void* scatter_index, hipStream_t stream);
+
 // float32 logits [R, V], temperature [R] (<= 0: greedy), uniform [R] in [0, 1) -> int32 out [R].
 int lle_sample_rows(const void* logits, const void* temperature, const void* uniform, void* out, int R, int V,
                     hipStream_t stream);

@@ -69,9 +69,14 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_chunks_kernel(const flo
 }
 
 // stage 2: grid rows, one wavefront: the first maximum among the chunks' winners
+// With `scatter_dst` the pick of row r also goes to scatter_dst[scatter_index[r]] (the token that
+// a request's slot decodes next, kept on the device for a step that is launched before the host
+// has read this one's picks).
 __global__ __launch_bounds__(LLE_WAVE) void argmax_final_kernel(const float* __restrict__ part_val,
                                                                 const int32_t* __restrict__ part_idx,
-                                                                int32_t* __restrict__ out, int chunks) {
+                                                                int32_t* __restrict__ out, int chunks,
+                                                                int32_t* __restrict__ scatter_dst = nullptr,
+                                                                const int32_t* __restrict__ scatter_index = nullptr) {
     __shared__ float s_val[1];
     __shared__ int s_idx[1];
     float best = -INFINITY;
@@ -85,19 +90,30 @@ __global__ __launch_bounds__(LLE_WAVE) void argmax_final_kernel(const float* __r
         }
     }
     block_argmax(best, best_i, s_val, s_idx);
-    if (threadIdx.x == 0) out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+    if (threadIdx.x == 0) {
+        const int pick = best_i == 0x7fffffff ? 0 : best_i;
+        out[blockIdx.x] = pick;
+        if (scatter_dst) scatter_dst[scatter_index[blockIdx.x]] = pick;
+    }
 }
 
-// `part_val`, `part_idx`: workspaces of R * chunks elements
-extern "C" int lle_argmax_rows(const void* logits, void* out, void* part_val, void* part_idx, int R, int V,
-                               int chunks, hipStream_t stream) {
+// `part_val`, `part_idx`: workspaces of R * chunks elements; `scatter_dst` (int32) and
+// `scatter_index` (int32 [R], in range of scatter_dst) both or neither: see argmax_final_kernel
+extern "C" int lle_argmax_rows_scatter(const void* logits, void* out, void* part_val, void* part_idx, int R, int V,
+                                       int chunks, void* scatter_dst, const void* scatter_index, hipStream_t stream) {
     if (R <= 0) return 0;
-    if (chunks <= 0 || chunks > 65535) return (int)hipErrorInvalidValue;
+    if (chunks <= 0 || chunks > 65535 || (scatter_dst == nullptr) != (scatter_index == nullptr))
+        return (int)hipErrorInvalidValue;
     argmax_chunks_kernel<<<dim3(R, chunks), ARGMAX_THREADS, 0, stream>>>((const float*)logits, (float*)part_val,
                                                                           (int32_t*)part_idx, V);
     argmax_final_kernel<<<R, LLE_WAVE, 0, stream>>>((const float*)part_val, (const int32_t*)part_idx, (int32_t*)out,
-                                                     chunks);
+                                                     chunks, (int32_t*)scatter_dst, (const int32_t*)scatter_index);
     LLE_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int lle_argmax_rows(const void* logits, void* out, void* part_val, void* part_idx, int R, int V,
+                               int chunks, hipStream_t stream) {
+    return lle_argmax_rows_scatter(logits, out, part_val, part_idx, R, V, chunks, nullptr, nullptr, stream);
 }
 
 // Chunks of a row: enough workgroups to stream a long row from all CUs.

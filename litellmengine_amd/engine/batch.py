@@ -51,6 +51,9 @@ class StepState:
     max_kv_len: int  # host-side bounds; they choose kernels, never results
     seqs: Optional[List[SeqInfo]]  # the same on the host (None inside a captured graph)
     scratch: dict = dataclasses.field(default_factory=dict)  # what parts make once per step and share
+    # int32, indexed by request slot: the token that the step before picked for a request, left on the
+    # device; a token id of -1 in `token_ids` stands for it (None: every id of the step is given)
+    token_feedback: Optional[torch.Tensor] = None
 
 
 @dataclasses.dataclass
@@ -73,26 +76,46 @@ class StepLayout:
 
 class _Staging:
     """Host buffers that the native layout writes into: pinned (page-locked) when a GPU will
-    read them, grown as needed and used again by the next step (the copy to the device has
-    ended when a step's arrays are used again)."""
+    read them, grown as needed and used again.  Three take turns: a step may be laid out while
+    the copy of the step before it to the device has not run yet (steps that are launched
+    ahead of the host's reading of their predecessor), and whoever launches ahead waits for
+    step k before laying out step k + 2."""
+
+    TURNS = 3
 
     def __init__(self):
         self.buffers = {}
+        self.copied = {}  # buffer -> event after the last copy out of it that was put on a stream
+        self.turn = 0
+        self.key = None
 
     def get(self, n: int, pinned: bool) -> torch.Tensor:
-        buf = self.buffers.get(pinned)
+        self.turn = (self.turn + 1) % self.TURNS
+        key = self.key = (pinned, self.turn)
+        done = self.copied.pop(key, None)
+        if done is not None:
+            done.synchronize()  # (long past, unless the caller put three steps on the stream without ever waiting)
+        buf = self.buffers.get(key)
         if buf is None or buf.numel() < n:
             size = max(1024, 1 << (max(1, n) - 1).bit_length())
             buf = torch.empty(size, dtype=torch.int32, pin_memory=pinned)
-            self.buffers[pinned] = buf
+            self.buffers[key] = buf
         return buf[:n]
+
+    def copy_enqueued(self) -> None:
+        """The buffer handed out last has a copy to the device waiting on the current stream."""
+        if self.key is not None and self.key[0]:
+            event = torch.cuda.Event()
+            event.record()
+            self.copied[self.key] = event
 
 
 _staging = _Staging()
+_update_staging = _Staging()
 
 
 def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, vocab_size: int = 0,
-                device=None, pad_to: int = 0, with_seqs: bool = True) -> StepLayout:
+                device=None, pad_to: int = 0, with_seqs: bool = True, allow_deferred: bool = False) -> StepLayout:
     """Lay the entries out flat and compute every token's page slot in every cache
     group (csrc/host.cpp does both).  Pages for the new lengths must already be there.
     `all_rows` asks for the logits of every row whatever the entries want; with
@@ -100,7 +123,9 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
     up to that many requests with single tokens that stand for nobody: they read the
     cache's spare table row and page (`cache.pad_slot`) and write nothing.  Without
     `with_seqs` the host-side list of the requests is left out (a step that runs as a graph
-    has no use for it, and it costs as much as everything else here)."""
+    has no use for it, and it costs as much as everything else here).  With `allow_deferred` a
+    token id of -1 is let through: it stands for the token that is still on the device
+    (StepState.token_feedback)."""
     S = len(entries)
     pad = max(0, pad_to - S)
     slots = array("i", [e.slot for e in entries])
@@ -141,9 +166,9 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
     handles = (ctypes.c_void_p * max(1, G))(*[g.native.handle for g in cache.groups])
     info = ctypes.c_int64(0)
     address = lambda a: a.buffer_info()[0]
-    code = lib.lle_layout_step(S, address(slots), address(past), address(q_len), address(tokens), int(vocab_size), R,
-                               address(rows), G, handles, pad, cache.pad_slot if pad else 0, host.data_ptr(),
-                               ctypes.byref(info))
+    code = lib.lle_layout_step(S, address(slots), address(past), address(q_len), address(tokens), int(vocab_size),
+                               int(allow_deferred), R, address(rows), G, handles, pad, cache.pad_slot if pad else 0,
+                               host.data_ptr(), ctypes.byref(info))
     if code == BAD_TOKEN:
         raise ValueError(f"token id {tokens[info.value]} outside [0, {vocab_size})")
     if code == NO_PAGE_AT_POSITION:
@@ -163,7 +188,8 @@ def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:
 
 
 def apply_table_updates(cache, device) -> None:
-    """Send the block-table entries made since the last step to the device tables."""
+    """Send the block-table entries made since the last step to the device tables (through a
+    pinned buffer and a copy that does not wait for the work already on the stream)."""
     updates = cache.take_table_updates()
     if not updates:
         return
@@ -171,7 +197,13 @@ def apply_table_updates(cache, device) -> None:
     for _, idx, pages in updates:
         flat += idx
         flat += pages
-    buf = torch.tensor(flat, dtype=torch.int32).to(device)  # a few entries a step
+    if torch.device(device).type == "cuda":
+        host = _update_staging.get(len(flat), True)
+        host.copy_(torch.tensor(flat, dtype=torch.int32))
+        buf = host.to(device, non_blocking=True)  # a few entries a step
+        _update_staging.copy_enqueued()
+    else:
+        buf = torch.tensor(flat, dtype=torch.int32)
     off = 0
     for g, idx, pages in updates:
         n = len(idx)
@@ -180,7 +212,7 @@ def apply_table_updates(cache, device) -> None:
 
 
 def state_on(buf: torch.Tensor, layout: StepLayout, cache, max_kv_len: Optional[int] = None,
-             with_seqs: bool = True) -> StepState:
+             with_seqs: bool = True, token_feedback: Optional[torch.Tensor] = None) -> StepState:
     """A StepState whose arrays are views of `buf` (which holds, or will hold,
     layout.flat); also points every cache group's slot mapping into it."""
     v = views_of(buf, layout.sizes())
@@ -191,12 +223,18 @@ def state_on(buf: torch.Tensor, layout: StepLayout, cache, max_kv_len: Optional[
         seq_slots=v[3], cu_tokens=v[4], kv_lens=v[5], logit_rows=v[6],
         min_q_len=layout.q_lens[0], max_q_len=layout.q_lens[1],
         max_kv_len=max_kv_len or layout.max_kv_len, seqs=layout.seqs if with_seqs else None,
+        token_feedback=token_feedback,
     )
 
 
-def build_step(entries: Sequence[StepEntry], cache, device, vocab_size: int = 0) -> StepState:
+def build_step(entries: Sequence[StepEntry], cache, device, vocab_size: int = 0, all_rows: bool = False,
+               token_feedback: Optional[torch.Tensor] = None) -> StepState:
     """Layout, one upload, views; also sends new block-table entries."""
-    layout = layout_step(entries, cache, vocab_size=vocab_size, device=device)
+    layout = layout_step(entries, cache, all_rows=all_rows, vocab_size=vocab_size, device=device,
+                         allow_deferred=token_feedback is not None)
     apply_table_updates(cache, device)
-    buf = layout.host.to(device) if torch.device(device).type != "cpu" else layout.host.clone()
-    return state_on(buf, layout, cache)
+    on_gpu = torch.device(device).type != "cpu"
+    buf = layout.host.to(device, non_blocking=True) if on_gpu else layout.host.clone()
+    if on_gpu:
+        _staging.copy_enqueued()
+    return state_on(buf, layout, cache, token_feedback=token_feedback)

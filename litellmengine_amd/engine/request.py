@@ -41,6 +41,9 @@ class Request:
     # appended and only the new tokens are run (finishing does not free in the reference,
     # src/engine/paged_generate_engine.cpp:386-395)
     keep_session: bool = False
+    # 1 while a token has been picked for the request on the device and the host has not read it
+    # yet (a step launched ahead): it counts as a token that is there but not cached
+    pending: int = 0
 
     def __post_init__(self):
         # a stream of its own: what a request draws does not depend on its batch mates
@@ -53,7 +56,12 @@ class Request:
     @property
     def extend_len(self) -> int:
         """Tokens not yet in the cache (include/engine/request.hpp:59-61)."""
-        return len(self.tokens) - self.cached_len
+        return len(self.tokens) + self.pending - self.cached_len
+
+    @property
+    def awaits_last_token(self) -> bool:
+        """The token on its way is the last one the request may generate: nothing more to run."""
+        return self.pending > 0 and len(self.generated) + self.pending >= self.max_new_tokens
 
     @property
     def remain_len(self) -> int:
@@ -65,7 +73,7 @@ class Request:
 
     def mark_forward_done(self, num_tokens: int) -> None:
         """src/engine/request_manager.cpp:190-213"""
-        if num_tokens < 0 or self.cached_len + num_tokens > len(self.tokens):
+        if num_tokens < 0 or self.cached_len + num_tokens > len(self.tokens) + self.pending:
             raise ValueError("mark_forward_done exceeds the request's tokens")
         self.cached_len += num_tokens
 

@@ -179,7 +179,7 @@ class Scheduler:
         or decode a chosen set (src/engine/paged_generate_engine.cpp:99-149, :182-341)."""
         budget = self.max_tokens_per_step
         chosen = None if only is None else set(only)
-        mine = [r for r in self.running if chosen is None or r.request_id in chosen]
+        mine = [r for r in self.running if (chosen is None or r.request_id in chosen) and not r.awaits_last_token]
         turn = lambda r: self._last_served.get(r.request_id, -1)
         decoding = sorted((r for r in mine if r.extend_len == 1), key=turn)
         prompts = [r for r in mine if r.extend_len > 1]
@@ -261,20 +261,36 @@ class Scheduler:
         """After the step ran: advance the caches' lengths, append the drawn tokens
         (one per portion with `samples`, in plan order), finish and free.
         Returns the requests that finished in this step."""
+        self.launched(plan)
+        return self.resolved(plan, sampled)
+
+    def launched(self, plan: Sequence[Portion]) -> None:
+        """The step of `plan` is on its way: its tokens count as cached."""
+        for p in plan:
+            p.request.mark_forward_done(p.num_tokens)
+
+    def resolved(self, plan: Sequence[Portion], sampled: Sequence[int]) -> List[Request]:
+        """The tokens that the step of `plan` drew are known (one per portion with `samples`, in
+        plan order): append them, finish and free.  A request that has finished or been released
+        since the step was launched (it ran one token past its end: the host learnt of the end a
+        step late) takes no token any more.  Returns the requests that finished."""
         done: List[Request] = []
         it = iter(sampled)
         for p in plan:
-            r = p.request
-            r.mark_forward_done(p.num_tokens)
-            if p.samples:
-                r.append_token(next(it))
-                if r.finished:
-                    self.running.remove(r)
-                    self._last_served.pop(r.request_id, None)
-                    if r.keep_session:
-                        self.parked.append(r)
-                    else:
-                        self.cache.release(r.slot)
-                        r.slot = -1
-                    done.append(r)
+            if not p.samples:
+                continue
+            r, token = p.request, next(it)
+            if r.status is not RequestStatus.RUNNING:
+                continue
+            r.pending = 0
+            r.append_token(token)
+            if r.finished:
+                self.running.remove(r)
+                self._last_served.pop(r.request_id, None)
+                if r.keep_session:
+                    self.parked.append(r)
+                else:
+                    self.cache.release(r.slot)
+                    r.slot = -1
+                done.append(r)
         return done

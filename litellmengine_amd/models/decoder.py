@@ -104,7 +104,7 @@ class DecoderLM:
         """Run the tokens of `step` (engine.batch.StepState) through the plan and
         return float32 logits [len(step.logit_rows), vocab]."""
         step.scratch.clear()  # per-step tables are made anew in every run (also when a graph is captured)
-        hidden = self.embedding.forward(step.token_ids)
+        hidden = self.embedding.forward(step.token_ids, step)
         delta = None
         last = len(self.plan) - 1
         for i, e in enumerate(self.plan):

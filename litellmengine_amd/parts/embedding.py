@@ -24,5 +24,9 @@ class Embedding(Part):
         self.ctx = ctx
         self.weight = weights[self.name].to(ctx.dtype).contiguous()
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, step=None) -> torch.Tensor:
+        """`step` (engine.batch.StepState): where it carries `token_feedback`, ids below zero are
+        the tokens that the step before left on the device for their requests."""
+        if step is not None and step.token_feedback is not None:
+            return self.ctx.ops.embedding(ids, self.weight, step.token_feedback, step.token_seq, step.seq_slots)
         return self.ctx.ops.embedding(ids, self.weight)

@@ -10,8 +10,23 @@ from tests.tiny import CONFIGS, make_model_dir, random_tokens
 from tests.torch_ops import TorchOps
 
 
+RUN_AHEAD = False
+
+
+@pytest.fixture(autouse=True, params=[False, True], ids=["step by step", "steps launched ahead"])
+def both_ways_of_stepping(request):
+    """Every test of this file runs twice: with each step's tokens read before the next step is
+    laid out, and with decode steps launched ahead of that reading (the device feeds a
+    request's pick to its next step; the host learns of an end-of-sequence token a step late)."""
+    global RUN_AHEAD
+    RUN_AHEAD = request.param
+    yield
+    RUN_AHEAD = False
+
+
 def cpu_engine(d, **kw):
     model = load_model(d, "float32", device="cpu", ops=TorchOps())
+    kw.setdefault("run_ahead", RUN_AHEAD)
     return LLMEngine(model, **kw)
 
 
@@ -116,6 +131,51 @@ def test_eos_is_appended_and_ends_the_request(tmp_path):
     eos = free[at]
     cut = free[: at + 1]
     assert cpu_engine(d, page_size=16, num_pages=8, max_requests=1).generate([p], 8, eos_token_id=eos) == [cut]
+
+
+def test_steps_launched_ahead_learn_of_an_end_a_step_late_and_change_nothing(tmp_path):
+    """Three greedy requests decode together; one meets its end-of-sequence token, one its token
+    limit, one goes on.  With steps launched ahead the host reads a step's tokens while the next
+    step is already on its way: the request that met its end ran one token too far (that token
+    is dropped, its position counts as cached), the one at its limit was not scheduled again;
+    the tokens are those of stepping one by one, a session goes on from there, a request that
+    arrives in between is served, and a request that is released while a step is on its way
+    takes no token any more."""
+    d = make_model_dir(tmp_path, "C")
+    cfg, w = plain.read_model_dir(d)
+    prompts = [random_tokens(n, 311, 70 + i) for i, n in enumerate((6, 11, 3))]
+    free = [plain.generate_greedy(p, w, cfg, 12) for p in prompts]
+    eos = free[0][4]  # request 0 ends with its fifth token (or earlier, if the token came before)
+    want0 = plain.generate_greedy(prompts[0], w, cfg, 12, eos=eos)
+    assert 1 < len(want0) < 12
+    outs = {}
+    for ahead in (False, True):
+        eng = cpu_engine(d, page_size=16, num_pages=12, max_requests=4, run_ahead=ahead)
+        a = eng.add_request(prompts[0], 12, eos_token_id=eos, keep_session=True)
+        b = eng.add_request(prompts[1], 7)
+        c = eng.add_request(prompts[2], 30)
+        late = None
+        while not (a.finished and b.finished):
+            eng.step()
+            if late is None and len(c.generated) >= 3:
+                late = eng.add_request(prompts[1][:5], 4)  # arrives while the others decode
+        assert a.generated == want0 and b.generated == free[1][:7]
+        # the session goes on: its history, more input, new tokens
+        more = random_tokens(4, 311, 99)
+        eng.append_input_tokens(a, more, 5)
+        while not a.finished:
+            eng.step()
+        assert a.generated == plain.generate_greedy(prompts[0] + want0 + more, w, cfg, 5)
+        eng.release_request(a)
+        while len(c.generated) + c.pending < 20:
+            eng.step()
+        eng.release_request(c)  # perhaps with a step of it on its way
+        eng.run_until_finished()
+        assert late.finished and late.generated == plain.generate_greedy(prompts[1][:5], w, cfg, 4)
+        assert c.generated == plain.generate_greedy(prompts[2], w, cfg, 30)[: len(c.generated)] and len(c.generated) >= 19
+        assert all(g.pool.num_held == 0 for g in eng.cache.groups) and eng.cache.num_free_slots == 4
+        outs[ahead] = (eng.num_steps_ahead, eng.num_steps)
+    assert outs[False][0] == 0 and outs[True][0] > 10, outs
 
 
 def test_temperature_draws_do_not_depend_on_the_batch(tmp_path):
@@ -446,7 +506,7 @@ def test_random_arrivals_small_pool_sessions_match_plain_gpu(tmp_path, seed, dty
     steps run through captured graphs, and the device tables hold rows of requests long gone."""
     d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
     model = load_model(d, dtype)
-    eng = LLMEngine(model, page_size=16, num_pages=14, max_requests=4, prefill_chunk=28, max_tokens_per_step=48)
+    eng = LLMEngine(model, page_size=16, num_pages=14, max_requests=4, prefill_chunk=28, max_tokens_per_step=48, run_ahead=RUN_AHEAD)
     assert eng.runner.use_graphs
     pre, ev = random_arrivals(eng, d, seed, 16, exact=dtype == "float32")
     print(f"random arrivals on the GPU, {dtype}, seed {seed}: {pre} preemptions, {ev} evictions")
@@ -461,7 +521,7 @@ def test_sessions_on_the_gpu(tmp_path, dtype):
     d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
     cfg, w = plain.read_model_dir(d)
     model = load_model(d, dtype)
-    eng = LLMEngine(model, page_size=16, num_pages=24, max_requests=3, prefill_chunk=20)
+    eng = LLMEngine(model, page_size=16, num_pages=24, max_requests=3, prefill_chunk=20, run_ahead=RUN_AHEAD)
     firsts = [random_tokens(n, 419, 70 + i) for i, n in enumerate((37, 9, 50))]
     mores = [random_tokens(n, 419, 80 + i) for i, n in enumerate((11, 3))]
     reqs = [eng.add_request(p, 6, keep_session=i < 2) for i, p in enumerate(firsts)]
@@ -514,7 +574,7 @@ def test_a_shrinking_batch_walks_through_few_graphs(tmp_path, dtype, max_graphs)
     d = make_model_dir(tmp_path, "D", dtype=torch.bfloat16)
     cfg, w = plain.read_model_dir(d)
     model = load_model(d, dtype)
-    eng = LLMEngine(model, page_size=16, num_pages=13 * 4, max_requests=13, max_tokens_per_step=512)
+    eng = LLMEngine(model, page_size=16, num_pages=13 * 4, max_requests=13, max_tokens_per_step=512, run_ahead=RUN_AHEAD)
     eng.runner.MAX_GRAPHS = max_graphs
     for wave in range(2):
         prompts = [random_tokens(5 + 2 * i, 419, 300 + 20 * wave + i) for i in range(13)]

@@ -23,8 +23,11 @@ class TorchOps:
     def __init__(self, compute_dtype=torch.float64):
         self.cd = compute_dtype
 
-    def embedding(self, ids, table):
-        return table[ids.long()].to(torch.float32)
+    def embedding(self, ids, table, feedback=None, token_seq=None, seq_slots=None):
+        ids = ids.long()
+        if feedback is not None:
+            ids = torch.where(ids < 0, feedback.long()[seq_slots.long()[token_seq.long()]], ids)
+        return table[ids].to(torch.float32)
 
     # the fused and sliced forms are the HIP kernels' own: this stand-in offers none of them
     def can_fold_norm(self, rows, width, dtype):
@@ -139,8 +142,11 @@ class TorchOps:
     def gate_up_silu(self, x, weight):
         return self.silu_mul(self.linear(x, weight))
 
-    def argmax(self, logits):
-        return torch.argmax(logits, dim=-1).to(torch.int32)  # torch returns the first maximum
+    def argmax(self, logits, scatter=None):
+        out = torch.argmax(logits, dim=-1).to(torch.int32)  # torch returns the first maximum
+        if scatter is not None:
+            scatter[0][scatter[1].long()] = out
+        return out
 
     def sample(self, logits, temperature, uniform):
         out = []
