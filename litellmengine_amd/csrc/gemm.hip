@@ -894,11 +894,25 @@ extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hi
 // The product AFTER a folded norm: X is the xw of lle_gemm_skinny_resid_bf16 and ss_part its
 // (16 or 32) x `parts` sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).
 // gated != 0: W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.
-// 1 <= M <= 32.
+// C is bfloat16, or float32 for a product that is not gated (an output head).  1 <= M <= 32.
+template <typename TC>
+static void launch_skinny_scaled(const bf16_t* x, const bf16_t* w, TC* c, int M, int N, int K, const NormFold& fold,
+                                 hipStream_t stream) {
+    if (launch_skinny_stream<false, true, TC>(x, w, c, M, N, K, fold, stream)) return;
+    const int threads = 16 * LLE_WAVE;
+    const int tr = skinny_tile_rows(N), blocks = (N + tr - 1) / tr;
+    if (M <= 16)
+        gemm_skinny_kernel<1, 1, false, false, true, TC, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+    else
+        gemm_skinny_kernel<2, 1, false, false, true, TC, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+}
+
 extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C, const void* ss_part, int parts,
-                                           float eps, int M, int N, int K, int gated, hipStream_t stream) {
+                                           float eps, int M, int N, int K, int gated, int out_dtype,
+                                           hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 32 || K % 8 != 0 || K <= 0 || parts <= 0 || (gated && N % 2 != 0)) return (int)hipErrorInvalidValue;
+    if (out_dtype != LLE_BF16 && !(out_dtype == LLE_F32 && !gated)) return (int)hipErrorInvalidValue;
     NormFold fold = {};
     fold.ss_in = (const float*)ss_part;
     fold.parts = parts;
@@ -907,19 +921,19 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
     const bf16_t* w = (const bf16_t*)W;
     bf16_t* c = (bf16_t*)C;
     const int threads = 16 * LLE_WAVE;
-    if (gated && launch_skinny_stream<true, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
-    } else if (!gated && launch_skinny_stream<false, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
-    } else {
-        const int rows = gated ? N / 2 : N;
-        const int tr = skinny_tile_rows(rows), blocks = (rows + tr - 1) / tr;
-        if (gated && M <= 16)
-            gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
-        else if (gated)
-            gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
-        else if (M <= 16)
-            gemm_skinny_kernel<1, 1, false, false, true, bf16_t, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+    if (!gated) {
+        if (out_dtype == LLE_F32)
+            launch_skinny_scaled<float>(x, w, (float*)C, M, N, K, fold, stream);
         else
-            gemm_skinny_kernel<2, 1, false, false, true, bf16_t, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+            launch_skinny_scaled<bf16_t>(x, w, c, M, N, K, fold, stream);
+    } else if (launch_skinny_stream<true, true, bf16_t>(x, w, c, M, N, K, fold, stream)) {
+    } else {
+        const int rows = N / 2;
+        const int tr = skinny_tile_rows(rows), blocks = (rows + tr - 1) / tr;
+        if (M <= 16)
+            gemm_skinny_kernel<1, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+        else
+            gemm_skinny_kernel<2, 2, true, false, true, bf16_t, 16, 2><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
     }
     LLE_RETURN_LAUNCH_STATUS();
 }

@@ -1,4 +1,4 @@
-// RMSNorm fused with the residual add.
+// RMSNorm fused with the residual add (and, for the first norm of a model, with the embedding).
 // Reference counterparts: rms_norm_forward_kernel (src/layers/rms_norm.cu:97-141)
 // and add_fp32_kernel (src/ops/add.cu:16-27), two launches there.
 //
@@ -165,6 +165,96 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
 
 // hidden += sums[0] + sums[1] + ... (float32 [slices][N][H], rows of hidden and of a slice alike), then
 // the norm as lle_add_rmsnorm; H a multiple of 4 up to 256 * 4 * NORM_CHUNKS
+// The first rows of the residual stream and their first norm in one launch: hidden[n] =
+// table[id(n)] as 32-bit (the embedding, src/layers/embedding.cu:75-87), out[n] its RMSNorm.
+// An id below zero stands for feedback[seq_slots[token_seq[n]]] (the token that the step before
+// picked for the row's request and left on the device), as in the embedding kernel itself.
+// VEC: rows of a multiple of 4 and at most 256 * 4 * NORM_CHUNKS elements, kept in registers.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void embedding_rmsnorm_kernel(const int32_t* __restrict__ ids,
+                                                                const T* __restrict__ table,
+                                                                float* __restrict__ hidden,
+                                                                const void* __restrict__ weight, int weight_dtype,
+                                                                T* __restrict__ out, int H, float eps,
+                                                                const int32_t* __restrict__ feedback,
+                                                                const int32_t* __restrict__ token_seq,
+                                                                const int32_t* __restrict__ seq_slots) {
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    int id = ids[n];
+    if (id < 0) id = feedback ? feedback[seq_slots[token_seq[n]]] : 0;
+    const T* row = table + (int64_t)id * H;
+    float* h = hidden + n * H;
+    T* o = out + n * H;
+    float ss = 0.f;
+    if constexpr (VEC) {
+        float4 v[NORM_CHUNKS], wv[NORM_CHUNKS];
+#pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                wv[k] = load_weight4(weight, i, weight_dtype);
+                v[k] = Quad<T>::load(row + i);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                *(float4*)(h + i) = v[k];
+                ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+            }
+        }
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+        for (int k = 0; k < NORM_CHUNKS; ++k) {
+            const int i = (k * 256 + threadIdx.x) * 4;
+            if (i < H) {
+                const float4 w = wv[k];
+                Quad<T>::store(o + i, make_float4(v[k].x * inv * w.x, v[k].y * inv * w.y, v[k].z * inv * w.z,
+                                                  v[k].w * inv * w.w));
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) {
+            const float v = to_f32<T>(row[i]);
+            h[i] = v;
+            ss += v * v;
+        }
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+        // (each thread reads back the elements that it wrote itself)
+        for (int i = threadIdx.x; i < H; i += blockDim.x)
+            o[i] = from_f32<T>(h[i] * inv * load_as_f32(weight, i, weight_dtype));
+    }
+}
+
+// ids int32 [N], table [V, H] and out [N, H] of `dtype`, hidden float32 [N, H]; `feedback`,
+// `token_seq` [N] and `seq_slots`: all three or none.  The host has checked the ids.
+extern "C" int lle_embedding_rmsnorm(const void* ids, const void* table, void* hidden, const void* weight,
+                                     int weight_dtype, void* out, int N, int H, float eps, int dtype,
+                                     const void* feedback, const void* token_seq, const void* seq_slots,
+                                     hipStream_t stream) {
+    if (N <= 0 || H <= 0) return 0;
+    if ((feedback != nullptr) != (token_seq != nullptr) || (feedback != nullptr) != (seq_slots != nullptr))
+        return (int)hipErrorInvalidValue;
+    const bool vec = H % 4 == 0 && H <= 256 * 4 * NORM_CHUNKS;
+#define LLE_EMBED_NORM(T, VEC)                                                                                  \
+    embedding_rmsnorm_kernel<T, VEC><<<N, 256, 0, stream>>>(                                                    \
+        (const int32_t*)ids, (const T*)table, (float*)hidden, weight, weight_dtype, (T*)out, H, eps,            \
+        (const int32_t*)feedback, (const int32_t*)token_seq, (const int32_t*)seq_slots)
+    if (dtype == LLE_F32) {
+        if (vec) LLE_EMBED_NORM(float, true); else LLE_EMBED_NORM(float, false);
+    } else if (dtype == LLE_BF16) {
+        if (vec) LLE_EMBED_NORM(bf16_t, true); else LLE_EMBED_NORM(bf16_t, false);
+    } else {
+        return (int)hipErrorInvalidValue;
+    }
+#undef LLE_EMBED_NORM
+    LLE_RETURN_LAUNCH_STATUS();
+}
+
 extern "C" int lle_add_rmsnorm_sums(void* hidden, const void* sums, int slices, int64_t slice_stride, const void* rows,
                                     const void* weight, int weight_dtype, void* out, int R, int H, float eps, int dtype,
                                     hipStream_t stream) {

@@ -115,6 +115,28 @@ class HipOps:
                   _ptr(token_seq) if feedback is not None else None, _ptr(seq_slots) if feedback is not None else None)
         return out
 
+    def embedding_rmsnorm(self, ids, table, weight, eps: float, feedback=None, token_seq=None, seq_slots=None):
+        """embedding() and the RMSNorm of its rows in one launch: (float32 [N, H] residual stream,
+        [N, H] normed rows in the table's type)."""
+        _dev(ids, "ids", torch.int32)
+        _dev(table, "embedding table")
+        _dev(weight, "norm weight")
+        _need(ids.dim() == 1 and table.dim() == 2, "embedding wants ids [N] and a table [V, H]")
+        N, H = ids.shape[0], table.shape[1]
+        _need(weight.shape == (H,), f"norm weight must be [{H}], is {list(weight.shape)}")
+        if feedback is not None:
+            for t, name in ((feedback, "feedback"), (token_seq, "token_seq"), (seq_slots, "seq_slots")):
+                _need(t is not None, "feedback, token_seq and seq_slots come together")
+                _dev(t, name, torch.int32)
+            _need(token_seq.shape == (N,), "token_seq must be [N]")
+        hidden = torch.empty((N, H), dtype=torch.float32, device=table.device)
+        out = torch.empty((N, H), dtype=table.dtype, device=table.device)
+        self._run("norm", "lle_embedding_rmsnorm", [_P, _P, _P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _P],
+                  _ptr(ids), _ptr(table), _ptr(hidden), _ptr(weight), dtype_code(weight.dtype), _ptr(out), N, H,
+                  float(eps), dtype_code(table.dtype), _ptr(feedback),
+                  _ptr(token_seq) if feedback is not None else None, _ptr(seq_slots) if feedback is not None else None)
+        return hidden, out
+
     # -- norms ---------------------------------------------------------------
     def add_rmsnorm(self, hidden, delta, weight, eps: float, out_dtype, rows=None) -> torch.Tensor:
         """hidden float32 [N, H] (+ delta [N, H] of out_dtype, or float32 partial sums
@@ -176,7 +198,7 @@ class HipOps:
         fn.argtypes, fn.restype = [_I], _I
         return int(fn(int(width)))
 
-    def _linear_folded(self, x, weight, fold, gated: bool):
+    def _linear_folded(self, x, weight, fold, gated: bool, out_dtype=torch.bfloat16):
         """The forms of the weight-streaming product around a folded norm: `x` a Prenormed
         (its row factors are applied to the result), `fold` a NormFold (the result goes
         into the residual stream and comes back as the next Prenormed)."""
@@ -196,9 +218,12 @@ class HipOps:
             _need(pre.sums.shape == (16 if M <= 16 else 32, parts) and pre.xw.shape[1] == K,
                   "sums of squares do not fit")
             _need(not gated or N % 2 == 0, "a gated weight has an even number of rows")
-            out = torch.empty((M, N // 2 if gated else N), dtype=torch.bfloat16, device=xin.device)
-            self._run("gemm", "lle_gemm_skinny_scaled_bf16", [_P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
-                      _ptr(xin), _ptr(weight), _ptr(out), _ptr(pre.sums), parts, float(pre.eps), M, N, K, int(gated))
+            _need(out_dtype == torch.bfloat16 or (out_dtype == torch.float32 and not gated),
+                  "the product after a folded norm writes bfloat16, or float32 where it is not gated")
+            out = torch.empty((M, N // 2 if gated else N), dtype=out_dtype, device=xin.device)
+            self._run("gemm", "lle_gemm_skinny_scaled_bf16", [_P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _P],
+                      _ptr(xin), _ptr(weight), _ptr(out), _ptr(pre.sums), parts, float(pre.eps), M, N, K, int(gated),
+                      dtype_code(out_dtype))
             return out
         _dev(fold.hidden, "hidden", torch.float32)
         _dev(fold.weight, "norm weight")
@@ -221,8 +246,9 @@ class HipOps:
         accumulate in 32-bit and write either result type.  `x` a Prenormed or `fold`
         a NormFold: see _linear_folded."""
         if fold is not None or isinstance(x, Prenormed):
-            _need(out_dtype in (None, torch.bfloat16), "a product beside a folded norm writes bfloat16")
-            return self._linear_folded(x, weight, fold, gated=False)
+            _need(out_dtype in (None, torch.bfloat16) or (fold is None and out_dtype == torch.float32),
+                  "a product that makes a folded norm's input writes bfloat16")
+            return self._linear_folded(x, weight, fold, gated=False, out_dtype=out_dtype or torch.bfloat16)
         _dev(x, "x")
         _dev(weight, "weight", x.dtype)
         M, K = x.shape

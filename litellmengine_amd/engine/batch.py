@@ -46,6 +46,7 @@ class StepState:
     cu_tokens: torch.Tensor  # int32 [S + 1] first row of each request, then N
     kv_lens: torch.Tensor  # int32 [S] cached length of each request after this step
     logit_rows: torch.Tensor  # int32 [R] rows whose logits are wanted
+    every_row_wanted: bool  # logit_rows is 0 .. N - 1 in order (known on the host)
     min_q_len: int
     max_q_len: int
     max_kv_len: int  # host-side bounds; they choose kernels, never results
@@ -68,6 +69,7 @@ class StepLayout:
     seqs: Optional[List[SeqInfo]]  # None when the caller asked for none
     max_kv_len: int
     q_lens: Tuple[int, int] = (1, 1)  # fewest and most tokens of a request in this step
+    every_row_wanted: bool = False  # the wanted rows are all rows, in order
 
     def sizes(self) -> List[int]:
         N, S, R = self.num_tokens, self.num_seqs, self.num_logit_rows
@@ -160,6 +162,7 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
         if with_seqs:
             seqs.extend(SeqInfo(cache.pad_slot, N + i, 1, 0) for i in range(pad))
     R = len(rows)
+    every_row = all_rows or (R == N + pad and all(r == i for i, r in enumerate(rows)))
     pinned = device is not None and torch.device(device).type == "cuda"
     host = _staging.get(3 * (N + pad) + 3 * (S + pad) + 1 + R + G * (N + pad), pinned)
     lib = host_library()
@@ -176,7 +179,8 @@ def layout_step(entries: Sequence[StepEntry], cache, all_rows: bool = False, voc
     if code != 0:
         raise ValueError(f"the step cannot be laid out: {lib.lle_error_string(code).decode()} (at {info.value})")
     q_lens = (min(q_len, default=1) if not pad else 1, max(q_len, default=1))
-    return StepLayout(host, N + pad, S + pad, R, G, seqs, max((p + n for p, n in zip(past, q_len)), default=1), q_lens)
+    return StepLayout(host, N + pad, S + pad, R, G, seqs, max((p + n for p, n in zip(past, q_len)), default=1), q_lens,
+                      every_row)
 
 
 def views_of(buf: torch.Tensor, sizes: Sequence[int]) -> List[torch.Tensor]:
@@ -221,6 +225,7 @@ def state_on(buf: torch.Tensor, layout: StepLayout, cache, max_kv_len: Optional[
     return StepState(
         num_tokens=layout.num_tokens, num_seqs=layout.num_seqs, token_ids=v[0], positions=v[1], token_seq=v[2],
         seq_slots=v[3], cu_tokens=v[4], kv_lens=v[5], logit_rows=v[6],
+        every_row_wanted=layout.every_row_wanted,
         min_q_len=layout.q_lens[0], max_q_len=layout.q_lens[1],
         max_kv_len=max_kv_len or layout.max_kv_len, seqs=layout.seqs if with_seqs else None,
         token_feedback=token_feedback,

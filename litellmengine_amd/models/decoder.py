@@ -16,7 +16,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import Block, BuildContext, Norm
+from ..parts.base import Block, BuildContext, Norm, Prenormed
 from ..parts.embedding import Embedding
 from ..parts.linear import Linear
 from ..weights.spec import TensorSpec
@@ -104,14 +104,20 @@ class DecoderLM:
         """Run the tokens of `step` (engine.batch.StepState) through the plan and
         return float32 logits [len(step.logit_rows), vocab]."""
         step.scratch.clear()  # per-step tables are made anew in every run (also when a graph is captured)
-        hidden = self.embedding.forward(step.token_ids, step)
-        delta = None
+        first_norm = self.blocks[self.plan[0].block].input_norm() if self.plan else None
+        if first_norm is not None:
+            hidden, delta = self.embedding.forward(step.token_ids, step, norm=first_norm)
+        else:
+            hidden, delta = self.embedding.forward(step.token_ids, step), None
         last = len(self.plan) - 1
         for i, e in enumerate(self.plan):
             # the norm that the next block starts with, if the products around it may do its work
-            next_norm = self.blocks[self.plan[i + 1].block].entry_norm() if i < last else None
+            if i < last:
+                next_norm = self.blocks[self.plan[i + 1].block].entry_norm()
+            else:  # the final norm, where the head's product can take its place (every row goes to the head)
+                next_norm = self.final_norm if step.every_row_wanted and not self.head.has_bias else None
             delta = self.blocks[e.block].forward(hidden, delta, step, caches.layer(i), next_norm=next_norm)
         if step.logit_rows.shape[0] == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=hidden.device)
-        x = self.final_norm.forward(hidden, delta, rows=step.logit_rows)
+        x = delta if isinstance(delta, Prenormed) else self.final_norm.forward(hidden, delta, rows=step.logit_rows)
         return self.head.forward(x, out_dtype=torch.float32)

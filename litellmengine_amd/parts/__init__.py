@@ -1,6 +1,6 @@
 from .attention import PagedAttention
 from .base import (Block, BuildContext, CacheField, CacheSpec, FeedForward, KVCacheSpec, Mixer, Norm, NormFold, Part,
-                   PartialSums, PositionEncoding, Prenormed, StateSpec)
+                   Normed, PartialSums, PositionEncoding, Prenormed, StateSpec)
 from .block import PreNormBlock
 from .embedding import Embedding
 from .feed_forward import GatedMLP
@@ -10,6 +10,6 @@ from .position import NoPositionEncoding, RotaryHalfSplit
 
 __all__ = [
     "Block", "BuildContext", "CacheField", "CacheSpec", "Embedding", "FeedForward", "GatedMLP", "KVCacheSpec", "Linear", "Mixer",
-    "NoPositionEncoding", "Norm", "NormFold", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
+    "NoPositionEncoding", "Norm", "NormFold", "Normed", "PagedAttention", "Part", "PartialSums", "PositionEncoding", "PreNormBlock", "Prenormed", "RMSNorm",
     "RotaryHalfSplit", "StateSpec",
 ]

@@ -135,6 +135,14 @@ class Prenormed:
 
 
 @dataclasses.dataclass
+class Normed:
+    """Rows that a block's first norm has been applied to already (by the kernel that made the
+    rows of the residual stream): the block takes `x` for its norm's result and adds nothing."""
+
+    x: torch.Tensor  # [N, width], activation type
+
+
+@dataclasses.dataclass
 class PartialSums:
     """A product that was taken in slices of its inner dimension and not added up yet:
     `sums` is float32 [slices, N, width], and the product is their sum in slice order.  Only a
@@ -156,10 +164,17 @@ class Norm(Part):
     `to_residual` may leave (`delta.total()` is the plain way to take them).
 
     fold(hidden) may return a NormFold when the step is small enough that the
-    products on both sides of the norm can do its work (None: call forward)."""
+    products on both sides of the norm can do its work (None: call forward).
+
+    of_embedding(ids, table, step) may return (hidden, normed rows) where a kernel makes the
+    rows of the residual stream from the embedding table and norms them in one go (None: the
+    embedding is taken on its own, then forward(hidden, None))."""
 
     def forward(self, hidden: torch.Tensor, delta: Optional[torch.Tensor], rows=None) -> torch.Tensor:
         raise NotImplementedError
+
+    def of_embedding(self, ids: torch.Tensor, table: torch.Tensor, step=None):
+        return None
 
     def fold(self, hidden: torch.Tensor) -> Optional[NormFold]:
         return None
@@ -226,11 +241,17 @@ class Block(Part):
 
     A block whose first norm can be folded into the products around it says so
     with entry_norm(); the model then passes the next block's as `next_norm`, and
-    the block may return a Prenormed made for that norm instead of a delta."""
+    the block may return a Prenormed made for that norm instead of a delta.
+
+    A block that begins with a norm of the residual stream and takes a `Normed` for
+    `delta` (the norm's result, made elsewhere) names that norm with input_norm()."""
 
     mixer: Mixer
 
     def entry_norm(self) -> Optional[Norm]:
+        return None
+
+    def input_norm(self) -> Optional[Norm]:
         return None
 
     def forward(self, hidden, delta, step, cache, next_norm=None):

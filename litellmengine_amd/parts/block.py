@@ -6,7 +6,7 @@ from __future__ import annotations
 from typing import Dict
 
 from ..weights.spec import TensorSpec
-from .base import Block, BuildContext, FeedForward, Mixer, Norm, Prenormed
+from .base import Block, BuildContext, FeedForward, Mixer, Norm, Normed, Prenormed
 
 
 class PreNormBlock(Block):
@@ -33,9 +33,16 @@ class PreNormBlock(Block):
     def entry_norm(self):
         return self.norm_in if self.mixer.folds_norm else None
 
+    def input_norm(self):
+        return self.norm_in
+
     def forward(self, hidden, delta, step, cache, next_norm=None):
-        # a Prenormed was made for norm_in by the block before: the add and the norm are done
-        x = delta if isinstance(delta, Prenormed) else self.norm_in.forward(hidden, delta)
+        if isinstance(delta, Prenormed):  # made for norm_in by the block before: the add and the norm are done
+            x = delta
+        elif isinstance(delta, Normed):  # norm_in's result, made together with the rows of `hidden`
+            x = delta.x
+        else:
+            x = self.norm_in.forward(hidden, delta)
         fold = self.norm_post.fold(hidden) if self.mixer.folds_norm and self.feed_forward.folds_norm else None
         if fold is not None:
             x = self.mixer.forward(x, step, cache, fold=fold)

@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from ..weights.spec import INIT_NORMAL, TensorSpec
-from .base import BuildContext, Part
+from .base import BuildContext, Normed, Part
 
 
 class Embedding(Part):
@@ -24,9 +24,16 @@ class Embedding(Part):
         self.ctx = ctx
         self.weight = weights[self.name].to(ctx.dtype).contiguous()
 
-    def forward(self, ids: torch.Tensor, step=None) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, step=None, norm=None):
         """`step` (engine.batch.StepState): where it carries `token_feedback`, ids below zero are
-        the tokens that the step before left on the device for their requests."""
+        the tokens that the step before left on the device for their requests.  With `norm` (the
+        parts.base.Norm that the first block begins with) the result is (rows, Normed or None):
+        the norm's result comes along where one kernel makes both."""
+        if norm is not None:
+            both = norm.of_embedding(ids, self.weight, step)
+            if both is not None:
+                return both[0], Normed(both[1])
+            return self.forward(ids, step), None
         if step is not None and step.token_feedback is not None:
             return self.ctx.ops.embedding(ids, self.weight, step.token_feedback, step.token_seq, step.seq_slots)
         return self.ctx.ops.embedding(ids, self.weight)

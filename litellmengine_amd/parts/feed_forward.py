@@ -13,9 +13,9 @@ from .linear import Linear
 
 
 class GatedMLP(FeedForward):
-    folds_norm = True
-
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
+        # the products that do a folded norm's work read their inner dimension eight elements at a time
+        self.folds_norm = intermediate_size % 8 == 0
         self.gate_up = Linear(
             [prefix + "gate_proj.weight", prefix + "up_proj.weight"], hidden_size, [intermediate_size] * 2
         )

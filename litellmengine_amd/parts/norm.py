@@ -28,6 +28,14 @@ class RMSNorm(Norm):
     def forward(self, hidden, delta, rows=None) -> torch.Tensor:
         return self.ctx.ops.add_rmsnorm(hidden, delta, self.weight, self.eps, self.ctx.dtype, rows)
 
+    def of_embedding(self, ids, table, step=None):
+        if table.dtype != self.ctx.dtype or table.shape[1] != self.size:
+            return None
+        if step is not None and step.token_feedback is not None:
+            return self.ctx.ops.embedding_rmsnorm(ids, table, self.weight, self.eps, step.token_feedback,
+                                                  step.token_seq, step.seq_slots)
+        return self.ctx.ops.embedding_rmsnorm(ids, table, self.weight, self.eps)
+
     def fold(self, hidden) -> Optional[NormFold]:
         if not self.ctx.ops.can_fold_norm(hidden.shape[0], self.size, self.ctx.dtype):
             return None

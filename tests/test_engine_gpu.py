@@ -199,9 +199,10 @@ ODD = [
     # one kv head for seven q heads, head size 64, page size 32, widths that are multiples of 2 only
     dict(num_hidden_layers=1, hidden_size=70, num_attention_heads=7, num_key_value_heads=1, head_dim=64,
          intermediate_size=94, vocab_size=333, rope_theta=1e6, rms_norm_eps=1e-5, tie_word_embeddings=False, page=32),
-    # head size 256, a window of 9 on every layer, page size 1
+    # head size 256, a window of 9 on every layer, page size 1; a width that the products around a folded
+    # norm take and a feed-forward width that they do not (a multiple of 4 only)
     dict(num_hidden_layers=2, hidden_size=64, num_attention_heads=2, num_key_value_heads=2, head_dim=256,
-         intermediate_size=72, vocab_size=50, rope_theta=1e4, rms_norm_eps=1e-6, tie_word_embeddings=False,
+         intermediate_size=76, vocab_size=50, rope_theta=1e4, rms_norm_eps=1e-6, tie_word_embeddings=False,
          sliding_window=9, layer_types=["sliding_attention", "sliding_attention"], page=1),
     # head size 96 (matrix cores, three 32-element steps), group of 3, page size 48
     dict(num_hidden_layers=2, hidden_size=96, num_attention_heads=6, num_key_value_heads=2, head_dim=96,

@@ -40,6 +40,33 @@ def test_embedding(dtype, H):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,wdtype", [(48, None), (1000, torch.float32), (4096, None), (4098, None), (9000, torch.float32)])
+def test_embedding_with_its_first_norm(dtype, H, wdtype):
+    """The rows of the table and their RMSNorm from one launch: the rows are the embedding's own
+    bit by bit, the normed rows what the norm kernel makes of them (and the float64 form); ids
+    below zero are looked up in the feedback table.  Row 5 is made large in one place, so a sum
+    over a part of the row shows."""
+    o = ops()
+    table = rnd((333, H), dtype, 1)
+    table[5, H - 1] = 30.0
+    w = (1 + 0.1 * rnd((H,), torch.float32, 4)).to(wdtype or dtype)
+    ids = torch.tensor([0, 332, 5, 5, 17], dtype=torch.int32).cuda()
+    hidden, x = o.embedding_rmsnorm(ids, table, w, 1e-3)
+    assert hidden.dtype == torch.float32 and x.dtype == dtype and x.shape == (5, H)
+    assert torch.equal(hidden, table[ids.long()].float())
+    want = REF.add_rmsnorm(hidden.clone(), None, w, 1e-3, dtype)
+    assert (x.double() - want.double()).abs().max() < tol(dtype, 4)
+    feedback = torch.tensor([7, 332, 5, 0], dtype=torch.int32).cuda()
+    seq_slots = torch.tensor([2, 0, 1], dtype=torch.int32).cuda()
+    token_seq = torch.tensor([0, 0, 1, 2, 2], dtype=torch.int32).cuda()
+    ids = torch.tensor([-1, 9, -1, 4, -1], dtype=torch.int32).cuda()
+    hidden, x = o.embedding_rmsnorm(ids, table, w, 1e-3, feedback, token_seq, seq_slots)
+    real = torch.tensor([5, 9, 7, 4, 332]).cuda()
+    assert torch.equal(hidden, table[real].float())
+    assert (x.double() - REF.add_rmsnorm(hidden.clone(), None, w, 1e-3, dtype).double()).abs().max() < tol(dtype, 4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,wdtype", [(80, None), (1000, torch.float32), (5120, None), (9000, None)])
 def test_add_rmsnorm(dtype, H, wdtype):
     N = 7
@@ -142,6 +169,13 @@ def test_norm_folded_into_products(wdtype, M, H, K, N):
             want = y
         assert got.dtype == torch.bfloat16 and got.shape == want.shape
         assert (got.double() - want).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+        if not gated:
+            # the same product left in float32 (an output head after the final norm): the bfloat16
+            # result is this one rounded, and against float64 only the operands' rounding is left
+            wide = o.linear(pre, w2, out_dtype=torch.float32)
+            assert wide.dtype == torch.float32 and wide.shape == want.shape
+            assert torch.equal(wide.to(torch.bfloat16), got)
+            assert (wide.double() - want).abs().max() < 1e-2 * max(1.0, want.abs().max().item())
         # against the unfolded kernels on the same numbers: the two differ by rounding only
         h2 = hidden.clone()
         x2 = o.add_rmsnorm(h2, o.linear(a, w1), nw, eps, torch.bfloat16)

@@ -29,6 +29,12 @@ class TorchOps:
             ids = torch.where(ids < 0, feedback.long()[seq_slots.long()[token_seq.long()]], ids)
         return table[ids].to(torch.float32)
 
+    def embedding_rmsnorm(self, ids, table, weight, eps, feedback=None, token_seq=None, seq_slots=None):
+        hidden = self.embedding(ids, table, feedback, token_seq, seq_slots)
+        x = hidden.to(self.cd)
+        x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.to(self.cd)
+        return hidden, x.to(table.dtype)
+
     # the fused and sliced forms are the HIP kernels' own: this stand-in offers none of them
     def can_fold_norm(self, rows, width, dtype):
         return False
