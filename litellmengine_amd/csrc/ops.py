@@ -12,6 +12,7 @@ import torch
 
 from ..parts.base import PartialSums, Prenormed
 from . import build
+from .tuning import ProductTuning
 from .limits import MAX_HEAD_DIM, MAX_SUMMED_NORM_WIDTH
 
 F32, BF16 = 0, 1
@@ -71,10 +72,11 @@ class HipOps:
 
     MAX_HEAD_DIM = MAX_HEAD_DIM
 
-    def __init__(self):
+    def __init__(self, tuning: Optional[ProductTuning] = None):
         if not torch.cuda.is_available():
             raise KernelError("litellmengine_amd needs a GPU: its kernels have no CPU form")
         self._fn = {}
+        self.tuning = tuning or ProductTuning()  # which kernel takes a product (never what it gives)
 
     # -- plumbing ---------------------------------------------------------
     def _get(self, lib: str, name: str, argtypes):
@@ -188,7 +190,7 @@ class HipOps:
     def can_fold_norm(self, rows: int, width: int, dtype) -> bool:
         """Whether an RMSNorm over `width` of a step of `rows` tokens can be done by the
         products before and after it (the weight-streaming kernel's few-rows forms)."""
-        most = 32 if width <= self.SKINNY_SMALL_WIDTH else self.SKINNY_MAX_ROWS
+        most = 32 if width <= self.tuning.skinny_small_width else self.tuning.skinny_max_rows
         return dtype == torch.bfloat16 and 0 < rows <= most and width % 8 == 0 and not self.force_library_gemm
 
     def norm_sum_parts(self, width: int) -> int:
@@ -266,7 +268,7 @@ class HipOps:
                     xs = x.view(M, slices, K // slices).permute(1, 0, 2)
                     ws = weight.view(N, slices, K // slices).permute(1, 2, 0)
                     return PartialSums(torch.bmm(xs, ws, out_dtype=torch.float32))
-            skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.SKINNY_MAX_ROWS
+            skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.tuning.skinny_max_rows
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
                 self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
@@ -276,7 +278,7 @@ class HipOps:
             return torch.mm(x, weight.t()) if out_dtype == torch.bfloat16 else torch.mm(x, weight.t(), out_dtype=out_dtype)
         _need(out_dtype == torch.float32, "a float32 product has a float32 result")
         out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-        if M <= self.SKINNY_F32_MAX_ROWS and K % 4 == 0 and not self.force_library_gemm:
+        if M <= self.tuning.skinny_f32_max_rows and K % 4 == 0 and not self.force_library_gemm:
             # few rows: W streamed once, float32 matrix instruction
             self._run("gemm", "lle_gemm_skinny_f32", [_P, _P, _P, _I, _I, _I, _P], _ptr(x), _ptr(weight), _ptr(out),
                       M, N, K)
@@ -308,7 +310,7 @@ class HipOps:
             return 0
         if N > MAX_SUMMED_NORM_WIDTH:  # the only reader of the partial sums (add_rmsnorm) takes no wider rows
             return 0
-        units = self.compute_units()
+        units, t = self.compute_units(), self.tuning
         groups = N // 64
         if groups > units // 2 or K % self.SLICED_UNIT != 0:  # (rows enough for the library's own tiles)
             return 0
@@ -319,15 +321,14 @@ class HipOps:
             if parts % slices != 0:
                 continue
             rounds = -(-groups * slices // units)
-            taken_in = (64 + rows) * (K // slices) * 2  # bytes of W and X through a CU, at about 29 GB/s
-            seconds = rounds * (3e-6 + taken_in / 29e9) + slices * M * N * 8 / 5e12
+            taken_in = (64 + rows) * (K // slices) * 2  # bytes of W and X through a CU
+            seconds = (rounds * (t.sliced_round_seconds + taken_in / t.cu_intake_bytes_per_s)
+                       + slices * M * N * 8 / t.partial_sums_bytes_per_s)
             if best == 0 or seconds < best_time:
                 best, best_time, best_fill = slices, seconds, groups * slices / (rounds * units)
-        if best_fill >= 0.85 or (K >= 2 * N and N * K >= self.SLICED_LONG_K_MIN_WEIGHT):
+        if best_fill >= t.sliced_min_fill or (K >= 2 * N and N * K >= t.sliced_long_k_min_weight):
             return best
         return 0
-
-    SLICED_LONG_K_MIN_WEIGHT = 1 << 23  # elements: below, a launch is as short as a launch can be either way
 
     def library_slices_for(self, M: int, N: int, K: int) -> int:
         """In how many slices of K the LIBRARY takes a product of more than 128 rows whose result is a
@@ -343,7 +344,7 @@ class HipOps:
         if N > MAX_SUMMED_NORM_WIDTH or N % 4 != 0:
             return 0
         tiles = -(-M // 256) * -(-N // 256)
-        slices = min(4, self.compute_units() // tiles)
+        slices = min(self.tuning.library_max_slices, self.compute_units() // tiles)
         while slices > 1 and K % (8 * slices) != 0:
             slices -= 1
         return slices if slices > 1 else 0
@@ -363,13 +364,7 @@ class HipOps:
                   M, N, K, slices)
         return out
 
-    # measured on MI355X: the weight-streaming kernels (with the norm folded into them) win up to 16
-    # rows, one tile of matrix-core columns, for every weight (batch 12 / 16 of the 8B sizes: 14 % / 10 %
-    # faster than the library products beside separate norms); up to 32 rows for small weights
-    SKINNY_MAX_ROWS = 16
-    SKINNY_F32_MAX_ROWS = 64  # the float32 twin: the plain-FMA kernel it replaces wastes its 64-row tiles on few rows
-    SKINNY_SMALL_WEIGHT = 1 << 25
-    SKINNY_SMALL_WIDTH = 2048  # models this narrow have small weights throughout: the norm is folded up to 32 rows
+    # (which of these kernels takes a product is decided by the numbers in self.tuning)
     force_library_gemm = False
     force_simt_gemm = False  # tests flip this to reach the plain-FMA kernel at sizes the matrix instruction takes
 
@@ -671,7 +666,7 @@ class HipOps:
         M, K = x.shape
         N2 = weight.shape[0]
         _need(weight.shape[1] == K and N2 % 2 == 0, f"weight {list(weight.shape)} does not fit x [{M}, {K}]")
-        few = M <= self.SKINNY_MAX_ROWS or (M <= 32 and N2 * K <= self.SKINNY_SMALL_WEIGHT)
+        few = M <= self.tuning.skinny_max_rows or (M <= 32 and N2 * K <= self.tuning.skinny_small_weight)
         if x.dtype == torch.bfloat16 and few and K % 8 == 0 and not self.force_library_gemm:
             out = torch.empty((M, N2 // 2), dtype=x.dtype, device=x.device)
             self._run("gemm", "lle_gemm_skinny_gated_bf16", [_P, _P, _P, _I, _I, _I, _P],
