@@ -796,14 +796,20 @@ static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M,
     return false;
 }
 
-// Rows of W per tile of the one-tile-per-workgroup kernel.  16 (a whole matrix-core tile) while the
-// tiles are at most one per CU or fill whole rounds of the CUs; otherwise as many as make the last
-// round full: with 320 tiles of 16 rows on 256 CUs a quarter of the CUs reads twice what the others
-// read and the launch lasts as long as two rounds, with 512 tiles of 10 rows every CU reads the same.
+// Rows of W per tile of the one-tile-per-workgroup kernel: as many as give every CU the same share.
+// More 16-row tiles than CUs: as many rows as make the last round full (with 320 tiles of 16 rows on
+// 256 CUs a quarter of the CUs reads twice what the others read and the launch lasts as long as two
+// rounds, with 512 tiles of 10 rows every CU reads the same).  Fewer tiles than CUs (narrow models):
+// lower tiles, down to 4 rows, so that every CU takes part: such a launch is short, and the share of
+// W that a workgroup has to wait for is what is left to shorten (measured at 16 rows of X: 1024 x 3072
+// 8.4 -> 7.3 us, 2048 x 6144 13.6 -> 12.1, 2560 x 9728 21.1 -> 18.9; tiles of 8 rows no better than of 4).
 static int skinny_tile_rows(int rows) {
     const int units = gemm_compute_units();
     const int tiles16 = (rows + 15) / 16;
-    if (tiles16 <= units) return 16;
+    if (tiles16 <= units) {
+        const int per_unit = (rows + units - 1) / units;
+        return per_unit < 4 ? 4 : (per_unit > 16 ? 16 : per_unit);
+    }
     const int rounds = (tiles16 + units - 1) / units;
     const int per_tile = (int)(((int64_t)rows + (int64_t)rounds * units - 1) / ((int64_t)rounds * units));
     return per_tile < 1 ? 1 : (per_tile > 16 ? 16 : per_tile);
