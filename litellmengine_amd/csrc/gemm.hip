@@ -901,16 +901,27 @@ extern "C" int lle_gemm_skinny_resid_bf16(const void* X, const void* W, void* hi
 // (16 or 32) x `parts` sums; the rows of the result are scaled by 1 / sqrt(sum / K + eps).
 // gated != 0: W is [2 I, K] and C [M, I] = silu(gate) * up as in lle_gemm_skinny_gated_bf16.
 // C is bfloat16, or float32 for a product that is not gated (an output head).  1 <= M <= 32.
+#ifndef SCALED_TILES_AT_32_ROWS
+#define SCALED_TILES_AT_32_ROWS 4
+#endif
 template <typename TC>
 static void launch_skinny_scaled(const bf16_t* x, const bf16_t* w, TC* c, int M, int N, int K, const NormFold& fold,
                                  hipStream_t stream) {
     if (launch_skinny_stream<false, true, TC>(x, w, c, M, N, K, fold, stream)) return;
     const int threads = 16 * LLE_WAVE;
     const int tr = skinny_tile_rows(N), blocks = (N + tr - 1) / tr;
-    if (M <= 16)
+    if (M <= 16) {
         gemm_skinny_kernel<1, 1, false, false, true, TC, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
-    else
+    } else if (N >= 16 * SCALED_TILES_AT_32_ROWS * gemm_compute_units()) {
+        // 17 to 32 rows of X are twice the bytes of a tile of W: with one tile a workgroup a product
+        // with many tiles (an output head) spends its time on X; several tiles share what they read of it
+        // (the head of the 0.6B sizes, 151936 x 1024, at 32 rows: 137.6 us with one tile, 126.8 with two, 112.1 with four)
+        constexpr int NT = SCALED_TILES_AT_32_ROWS;
+        gemm_skinny_kernel<2, NT, false, false, true, TC, 16, 4 / NT>
+            <<<(N + 16 * NT - 1) / (16 * NT), threads, 0, stream>>>(x, w, c, M, N, K, 16, fold);
+    } else {
         gemm_skinny_kernel<2, 1, false, false, true, TC, 16, 4><<<blocks, threads, 0, stream>>>(x, w, c, M, N, K, tr, fold);
+    }
 }
 
 extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C, const void* ss_part, int parts,

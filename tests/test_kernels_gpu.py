@@ -131,6 +131,8 @@ def test_gate_up_silu(dtype, M, I, K):
                                      (6, 4096, 256, 8189), (1, 4096, 128, 12288), (16, 4096, 256, 6151), (11, 5120, 128, 260),
                                      (7, 24, 8, 6), (16, 1024, 2048, 3072), (13, 520, 96, 70), (32, 1024, 2048, 3072),
                                      (17, 72, 40, 22), (29, 2048, 512, 128),
+                                     # 17 to 32 rows against so many tiles of W that a workgroup takes several (an output head)
+                                     (32, 1024, 128, 20000), (19, 520, 64, 16387),
                                      # more tiles than CUs, no whole rounds: tiles of fewer than 16 rows
                                      (9, 4600, 64, 4700), (16, 5120, 128, 5000), (3, 6152, 40, 4099)])
 def test_norm_folded_into_products(wdtype, M, H, K, N):
