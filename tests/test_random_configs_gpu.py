@@ -19,8 +19,9 @@ from tests.trace_util import (TraceBuilder, changing_portions, check_dumps, mixe
 
 pytestmark = pytest.mark.gpu
 
-# about five times the worst error seen over 240 such draws (float32 1.8e-6, sharpened 1.0e-5; bfloat16 8.9e-3)
-TOL = {"float32": 1e-5, "float32 sharpened": 5e-5, "bfloat16": 4e-2}
+# float32: about five times the worst error seen over 240 such draws (1.8e-6, sharpened 1.0e-5);
+# bfloat16: the tolerance of the fixed configurations' traces (the worst of those draws was 8.9e-3)
+TOL = {"float32": 1e-5, "float32 sharpened": 5e-5, "bfloat16": 2e-2}
 
 
 def draw(seed: int):
