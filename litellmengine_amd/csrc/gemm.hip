@@ -589,7 +589,12 @@ extern "C" int lle_gemm_mid_slices_bf16(const void* X, const void* W, void* out,
 // and written out.  X is read once per workgroup instead of once per tile, and the sums of
 // the folded norm are added up once.
 // ---------------------------------------------------------------------------------
-template <bool GATED, bool SCALED, int XS, typename TC>
+// MT = 2: up to 32 rows of X (two tiles of matrix-core columns), where all of X that a wavefront
+// needs still fits its registers (XS <= 2: narrow models, the only ones whose norms are folded at
+// more than 16 rows);
+// the head of the 0.6B sizes (151936 x 1024) at 32 rows: 73.6 us, against 112.1 for the
+// one-tile-per-workgroup kernel with four tiles a workgroup and 66.8 at 16 rows.
+template <bool GATED, bool SCALED, int XS, typename TC, int MT = 1>
 __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X,
                                                                               const bf16_t* __restrict__ W,
                                                                               TC* __restrict__ C, int M, int N, int K,
@@ -598,8 +603,9 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     constexpr int NT = GATED ? 2 : 1;
     constexpr int SS = (XS % 2 == 0 && XS <= 6) ? 2 : 1;  // steps of a set (one where X takes most of the registers)
     constexpr int SPT = XS / SS;             // sets of a tile
-    __shared__ float s_acc[2][WAVES][NT][16][17];  // tiles take the two halves in turn: one barrier a tile
-    __shared__ float s_inv[16];
+    static_assert(MT == 1 || (MT == 2 && XS <= 2), "two tiles of X rows only while X fits the registers");
+    __shared__ float s_acc[2][WAVES][NT][MT][16][17];  // tiles take the two halves in turn: one barrier a tile
+    __shared__ float s_inv[16 * MT];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
     const int rows = GATED ? N / 2 : N;
@@ -643,60 +649,72 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     aim();
     load(sets[0]);
     // rows of X beyond M are never written back, so their lanes may read any valid row
-    gbf16x8 x0[XS], x1[XS];
-    {
-        const bf16_t* xp = X + (int64_t)min(r16, M - 1) * K + 16 * c + wave * SK_KSTEP;
+    gbf16x8 x0[MT][XS], x1[MT][XS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const bf16_t* xp = X + (int64_t)min(16 * mt + r16, M - 1) * K + 16 * c + wave * SK_KSTEP;
 #pragma unroll
         for (int j = 0; j < XS; ++j) {
-            x0[j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP));
-            x1[j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP) + 8);
+            x0[mt][j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP));
+            x1[mt][j] = *(const gbf16x8*)(xp + j * (WAVES * SK_KSTEP) + 8);
         }
     }
     if (SCALED) {
-        // the row factors of the folded norm: wavefront w adds up the parts of row w, four loads at a time
-        const float* in = fold.ss_in + (int64_t)wave * fold.parts;
-        float part = 0.f;
-        for (int p0 = lane; p0 < fold.parts; p0 += 4 * LLE_WAVE) {
-            float v[4];
+        // the row factors of the folded norm: wavefront w adds up the parts of row w (and of row
+        // 16 + w), four loads at a time
 #pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = in[min(p0 + i * LLE_WAVE, fold.parts - 1)];
+        for (int mt = 0; mt < MT; ++mt) {
+            const float* in = fold.ss_in + (int64_t)(16 * mt + wave) * fold.parts;
+            float part = 0.f;
+            for (int p0 = lane; p0 < fold.parts; p0 += 4 * LLE_WAVE) {
+                float v[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) part += p0 + i * LLE_WAVE < fold.parts ? v[i] : 0.f;
+                for (int i = 0; i < 4; ++i) v[i] = in[min(p0 + i * LLE_WAVE, fold.parts - 1)];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) part += p0 + i * LLE_WAVE < fold.parts ? v[i] : 0.f;
+            }
+            part = wave_sum(part);
+            if (lane == 0) s_inv[16 * mt + wave] = 1.0f / sqrtf(part / (float)K + fold.eps);
         }
-        part = wave_sum(part);
-        if (lane == 0) s_inv[wave] = 1.0f / sqrtf(part / (float)K + fold.eps);
     }
-    gf32x4 acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+    gf32x4 acc_g[MT], acc_u[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc_g[mt] = acc_u[mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const Set& set, int j) {
 #pragma unroll
-        for (int i = 0; i < SS; ++i) {
-            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g0[i], x0[j + i], acc_g, 0, 0, 0);
-            acc_g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g1[i], x1[j + i], acc_g, 0, 0, 0);
-            if (GATED) {
-                acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u0[i], x0[j + i], acc_u, 0, 0, 0);
-                acc_u = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u1[i], x1[j + i], acc_u, 0, 0, 0);
+        for (int i = 0; i < SS; ++i)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g0[i], x0[mt][j + i], acc_g[mt], 0, 0, 0);
+                acc_g[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.g1[i], x1[mt][j + i], acc_g[mt], 0, 0, 0);
+                if (GATED) {
+                    acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u0[i], x0[mt][j + i], acc_u[mt], 0, 0, 0);
+                    acc_u[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(set.u1[i], x1[mt][j + i], acc_u[mt], 0, 0, 0);
+                }
             }
-        }
     };
     int half = 0;
     auto finish_tile = [&](int tile) {
-        // lane holds C^T[n = 4c + i][m = r16]
+        // lane holds C^T[n = 4c + i][m = 16 mt + r16]
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            s_acc[half][wave][0][4 * c + i][r16] = acc_g[i];
-            if (GATED) s_acc[half][wave][NT - 1][4 * c + i][r16] = acc_u[i];
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s_acc[half][wave][0][mt][4 * c + i][r16] = acc_g[mt][i];
+                if (GATED) s_acc[half][wave][NT - 1][mt][4 * c + i][r16] = acc_u[mt][i];
+            }
+            acc_g[mt] = acc_u[mt] = gf32x4{0.f, 0.f, 0.f, 0.f};
         }
-        acc_g = acc_u = gf32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
-        if (threadIdx.x < 256) {
+        if (threadIdx.x < 256 * MT) {
             const int m = threadIdx.x / 16, n = threadIdx.x % 16;
             const int64_t col = (int64_t)tile_begin(tile) + n;
             if (m < M && col < tile_end(tile)) {
                 float g = 0.f, u = 0.f;
 #pragma unroll
                 for (int w = 0; w < WAVES; ++w) {
-                    g += s_acc[half][w][0][n][m];
-                    if (GATED) u += s_acc[half][w][NT - 1][n][m];
+                    g += s_acc[half][w][0][m / 16][n][m % 16];
+                    if (GATED) u += s_acc[half][w][NT - 1][m / 16][n][m % 16];
                 }
                 if (SCALED) {
                     g *= s_inv[m];
@@ -761,12 +779,23 @@ static int gemm_compute_units() {
 template <bool GATED, bool SCALED, typename TC>
 static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M, int N, int K,
                                  const NormFold& fold, hipStream_t stream) {
-    if (M > 16 || K % (SK_KSTEP * 16) != 0) return false;
+    if (M > 32 || K % (SK_KSTEP * 16) != 0) return false;
     const int rows = GATED ? N / 2 : N;
     const int units = gemm_compute_units();
     const int share = (rows + units - 1) / units;
     if (share <= 16) return false;
     const int blocks = (rows + share - 1) / share;
+    if (M > 16) {  // two tiles of X rows: while all of X that a wavefront needs fits its registers
+        if (K == SK_KSTEP * 16) {
+            gemm_skinny_stream_kernel<GATED, SCALED, 1, TC, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
+            return true;
+        }
+        if (K == 2 * SK_KSTEP * 16) {
+            gemm_skinny_stream_kernel<GATED, SCALED, 2, TC, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
+            return true;
+        }
+        return false;
+    }
 #define LLE_STREAM_CASE(XSV)                                                                                          \
     case XSV:                                                                                                         \
         gemm_skinny_stream_kernel<GATED, SCALED, XSV, TC><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, \
