@@ -268,7 +268,9 @@ class HipOps:
                     xs = x.view(M, slices, K // slices).permute(1, 0, 2)
                     ws = weight.view(N, slices, K // slices).permute(1, 2, 0)
                     return PartialSums(torch.bmm(xs, ws, out_dtype=torch.float32))
-            skinny = K % 8 == 0 and not self.force_library_gemm and M <= self.tuning.skinny_max_rows
+            skinny = K % 8 == 0 and not self.force_library_gemm and (
+                M <= self.tuning.skinny_max_rows
+                or (M <= 32 and K <= self.tuning.skinny_small_width and N * K <= self.tuning.skinny_small_weight))
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
                 self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],
