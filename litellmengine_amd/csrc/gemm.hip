@@ -603,7 +603,7 @@ __global__ __launch_bounds__(16 * LLE_WAVE, 4) void gemm_skinny_stream_kernel(co
     constexpr int NT = GATED ? 2 : 1;
     constexpr int SS = (XS % 2 == 0 && XS <= 6) ? 2 : 1;  // steps of a set (one where X takes most of the registers)
     constexpr int SPT = XS / SS;             // sets of a tile
-    static_assert(MT == 1 || (MT == 2 && XS <= 2), "two tiles of X rows only while X fits the registers");
+    static_assert(MT == 1 || (MT == 2 && (XS <= 2 || (!GATED && XS <= 4))), "two tiles of X rows only while X fits the registers");
     __shared__ float s_acc[2][WAVES][NT][MT][16][17];  // tiles take the two halves in turn: one barrier a tile
     __shared__ float s_inv[16 * MT];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
@@ -793,6 +793,16 @@ static bool launch_skinny_stream(const bf16_t* X, const bf16_t* W, TC* C, int M,
         if (K == 2 * SK_KSTEP * 16) {
             gemm_skinny_stream_kernel<GATED, SCALED, 2, TC, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
             return true;
+        }
+        if constexpr (!GATED) {
+            if (K == 3 * SK_KSTEP * 16) {
+                gemm_skinny_stream_kernel<GATED, SCALED, 3, TC, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
+                return true;
+            }
+            if (K == 4 * SK_KSTEP * 16) {
+                gemm_skinny_stream_kernel<GATED, SCALED, 4, TC, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(X, W, C, M, N, K, share, fold);
+                return true;
+            }
         }
         return false;
     }

@@ -268,9 +268,13 @@ class HipOps:
                     xs = x.view(M, slices, K // slices).permute(1, 0, 2)
                     ws = weight.view(N, slices, K // slices).permute(1, 2, 0)
                     return PartialSums(torch.bmm(xs, ws, out_dtype=torch.float32))
+            t = self.tuning
             skinny = K % 8 == 0 and not self.force_library_gemm and (
-                M <= self.tuning.skinny_max_rows
-                or (M <= 32 and K <= self.tuning.skinny_small_width and N * K <= self.tuning.skinny_small_weight))
+                M <= t.skinny_max_rows
+                or (M <= 32 and K <= t.skinny_small_width and N * K <= t.skinny_small_weight)
+                # 17 to 32 rows against a weight with many rows for every CU: the streaming kernel with two
+                # tiles of X rows in its registers (K a multiple of 1024 up to 4096)
+                or (M <= 32 and K % 1024 == 0 and K <= 4096 and N >= t.stream_32_rows_min_share * self.compute_units()))
             if skinny:
                 out = torch.empty((M, N), dtype=out_dtype, device=x.device)
                 self._run("gemm", "lle_gemm_skinny_bf16", [_P, _P, _P, _I, _I, _I, _I, _P],

@@ -20,6 +20,11 @@ class ProductTuning:
     # is then as short as a launch can be, and one launch with the norm in it beats two
     skinny_small_weight: int = 1 << 25
     skinny_small_width: int = 2048
+    # 17 to 32 rows: the weight-streaming kernel (two tiles of X rows in its registers, K up to 4096)
+    # takes a plain product whose weight has at least this many rows for every CU (gate_up and the
+    # head of the 8B sizes: 41-43 against the library's 49 us, 239-250 against 270; qkv, 24 rows a CU,
+    # is the library's: 15-17 against 15 us)
+    stream_32_rows_min_share: int = 64
     # the float32 twin takes up to this many rows (the tiled float32 kernel wastes its 64-row tiles on fewer)
     skinny_f32_max_rows: int = 64
     # the sliced product (17 to 128 rows) is taken where its workgroups fill at least this share

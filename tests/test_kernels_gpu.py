@@ -326,6 +326,54 @@ def test_streaming_products_at_every_width(M, K):
     assert (got.double() - wantn).abs().max() < 2e-2 * max(1.0, wantn.abs().max().item())
 
 
+@pytest.mark.parametrize("K", [1024, 2048, 3072, 4096])
+@pytest.mark.parametrize("M", [17, 25, 32])
+def test_streaming_products_with_two_tiles_of_rows(M, K):
+    """17 to 32 rows of X in the weight-streaming forms: plain (both result types) against a weight
+    with many rows for every CU at every K they take, and, at the widths of narrow models, gated
+    and after a folded norm; against float64.  Row 16 of X is made large, so a second tile of rows
+    that is dropped or read twice shows, and W is made of rows that tell their own number."""
+    from litellmengine_amd.parts import NormFold
+
+    o = ops()
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    x = rnd((M, K), torch.bfloat16, 71)
+    x[16] *= 4.0
+    N = o.tuning.stream_32_rows_min_share * units + 16 * 5 + 7
+    w = rnd((N, K), torch.bfloat16, 72, 0.05)
+    w[:, 0] = (torch.arange(N) % 64).to(torch.bfloat16) / 16
+    want = x.double() @ w.double().t()
+    lim = 2e-2 * max(1.0, want.abs().max().item())
+    for out_dtype in (torch.bfloat16, torch.float32):
+        got = o.linear(x, w, out_dtype)
+        assert (got.double() - want).abs().max() < (lim if out_dtype == torch.bfloat16 else lim / 100)
+    if K > 2048:
+        return
+    assert o.can_fold_norm(M, K, torch.bfloat16)
+    n = 17 * units + 16 * 5 + 7  # more than one tile per CU
+    wg = rnd((2 * n, K), torch.bfloat16, 73, 0.05)
+    y = x.double() @ wg.double().t()
+    wantg = torch.nn.functional.silu(y[:, :n]) * y[:, n:]
+    got = o.gate_up_silu(x, wg)
+    assert (got.double() - wantg).abs().max() < 2e-2 * max(1.0, wantg.abs().max().item())
+    a = rnd((M, 64), torch.bfloat16, 74)
+    w1 = rnd((K, 64), torch.bfloat16, 75, 0.2)
+    hidden = rnd((M, K), torch.float32, 76, 1.5)
+    hidden[16] *= 3.0
+    nw = (1 + 0.3 * rnd((K,), torch.float32, 77)).to(torch.bfloat16)
+    pre = o.linear(a, w1, fold=NormFold(hidden, nw, 1e-3))
+    h = hidden.double()
+    normed = h * torch.rsqrt((h ** 2).mean(1, keepdim=True) + 1e-3) * nw.double()
+    for weight, gated in ((w[: 17 * units + 87], False), (wg, True)):
+        yn = normed @ weight.double().t()
+        wantn = torch.nn.functional.silu(yn[:, :n]) * yn[:, n:] if gated else yn
+        got = o.gate_up_silu(pre, weight) if gated else o.linear(pre, weight.contiguous())
+        assert (got.double() - wantn).abs().max() < 2e-2 * max(1.0, wantn.abs().max().item())
+        if not gated:
+            wide = o.linear(pre, weight.contiguous(), out_dtype=torch.float32)
+            assert (wide.double() - wantn).abs().max() < 1e-2 * max(1.0, wantn.abs().max().item())
+
+
 def test_silu_mul_reference_vector():
     # tests/test_silu_and_mul.cpp:48-56
     g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])
