@@ -1004,12 +1004,15 @@ extern "C" int lle_gemm_skinny_scaled_bf16(const void* X, const void* W, void* C
 template <int MT, int SK_WAVES, int UNROLL>
 __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_f32_kernel(const float* __restrict__ X,
                                                                              const float* __restrict__ W,
-                                                                             float* __restrict__ C, int M, int N, int K) {
+                                                                             float* __restrict__ C, int M, int N, int K,
+                                                                             int tile_rows) {
+    // `tile_rows` (at most 16) rows of W per workgroup, as in the bfloat16 kernel (skinny_tile_rows):
+    // the lanes past them read the tile's last row again and write nothing
     __shared__ float s_acc[SK_WAVES][MT][16][17];
     const int wave = threadIdx.x / LLE_WAVE, lane = threadIdx.x % LLE_WAVE;
     const int c = lane / 16, r16 = lane % 16;
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
-    const float* wp = W + min(n0 + r16, (int64_t)N - 1) * K + 4 * c;
+    const int64_t n0 = (int64_t)blockIdx.x * tile_rows;
+    const float* wp = W + min(n0 + min(r16, tile_rows - 1), (int64_t)N - 1) * K + 4 * c;
     // rows of X beyond M are never written back, so their lanes may read any valid row
     const float* xp[MT];
 #pragma unroll
@@ -1060,7 +1063,7 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_f32_kernel(con
     for (int idx = threadIdx.x; idx < MT * 256; idx += blockDim.x) {
         const int mt = idx / 256, m = (idx / 16) % 16, n = idx % 16;
         const int64_t row = 16 * mt + m, col = n0 + n;
-        if (row >= M || col >= N) continue;
+        if (row >= M || col >= N || n >= tile_rows) continue;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < SK_WAVES; ++w) sum += s_acc[w][mt][n][m];
@@ -1072,15 +1075,15 @@ __global__ __launch_bounds__(SK_WAVES* LLE_WAVE) void gemm_skinny_f32_kernel(con
 extern "C" int lle_gemm_skinny_f32(const void* X, const void* W, void* C, int M, int N, int K, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K % 4 != 0 || K <= 0) return (int)hipErrorInvalidValue;
-    const int blocks = (N + 15) / 16;
+    const int tr = skinny_tile_rows(N), blocks = (N + tr - 1) / tr;
     const float* x = (const float*)X;
     const float* w = (const float*)W;
     float* c = (float*)C;
     switch ((M + 15) / 16) {
-        case 1: gemm_skinny_f32_kernel<1, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
-        case 2: gemm_skinny_f32_kernel<2, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
-        case 3: gemm_skinny_f32_kernel<3, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
-        default: gemm_skinny_f32_kernel<4, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K); break;
+        case 1: gemm_skinny_f32_kernel<1, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K, tr); break;
+        case 2: gemm_skinny_f32_kernel<2, 16, 4><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K, tr); break;
+        case 3: gemm_skinny_f32_kernel<3, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K, tr); break;
+        default: gemm_skinny_f32_kernel<4, 16, 2><<<blocks, 16 * LLE_WAVE, 0, stream>>>(x, w, c, M, N, K, tr); break;
     }
     LLE_RETURN_LAUNCH_STATUS();
 }
