@@ -374,6 +374,50 @@ def test_streaming_products_with_two_tiles_of_rows(M, K):
             assert (wide.double() - wantn).abs().max() < 1e-2 * max(1.0, wantn.abs().max().item())
 
 
+@pytest.mark.parametrize("M", [3, 16, 24, 32, 40, 100, 300])
+def test_the_numbers_that_choose_a_kernel_change_no_result(M):
+    """ProductTuning decides which kernel takes a product, never what it gives: with every
+    threshold pushed to one end and to the other (the library for everything it may take; the
+    weight-streaming and sliced kernels for everything they take), plain and gated products and
+    a product that leaves its result as a delta of the residual stream agree with float64."""
+    import dataclasses
+
+    from litellmengine_amd.csrc.ops import HipOps
+    from litellmengine_amd.csrc.tuning import ProductTuning
+
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    K, N, I = 2048, 64 * units + 64, 1024
+    x = rnd((M, K), torch.bfloat16, 81)
+    w = rnd((N, K), torch.bfloat16, 82, 0.05)
+    wg = rnd((2 * I, K), torch.bfloat16, 83, 0.05)
+    wd = rnd((K, 4 * K), torch.bfloat16, 84, 0.05)  # K at least twice N: a candidate for slices
+    xd = rnd((M, 4 * K), torch.bfloat16, 85)
+    want = x.double() @ w.double().t()
+    y = x.double() @ wg.double().t()
+    want_g = torch.nn.functional.silu(y[:, :I]) * y[:, I:]
+    want_d = xd.double() @ wd.double().t()
+    base = ProductTuning()
+    ends = [
+        base,
+        dataclasses.replace(base, skinny_max_rows=0, skinny_small_weight=0, skinny_small_width=0,
+                            stream_32_rows_min_share=1 << 30, sliced_min_fill=2.0, sliced_long_k_min_weight=1 << 62,
+                            library_max_slices=1),
+        dataclasses.replace(base, skinny_small_weight=1 << 62, skinny_small_width=1 << 30, stream_32_rows_min_share=1,
+                            sliced_min_fill=0.0, sliced_long_k_min_weight=0),
+    ]
+    for tuning in ends:
+        o = HipOps(tuning=tuning)
+        got = o.linear(x, w)
+        assert (got.double() - want).abs().max() < 2e-2 * max(1.0, want.abs().max().item())
+        got = o.linear(x, w, torch.float32)
+        assert (got.double() - want).abs().max() < 2e-4 * max(1.0, want.abs().max().item())
+        got = o.gate_up_silu(x, wg)
+        assert (got.double() - want_g).abs().max() < 2e-2 * max(1.0, want_g.abs().max().item())
+        delta = o.linear(xd, wd, sums_ok=True)
+        total = delta.total() if hasattr(delta, "total") else delta
+        assert (total.double() - want_d).abs().max() < 2e-2 * max(1.0, want_d.abs().max().item())
+
+
 def test_silu_mul_reference_vector():
     # tests/test_silu_and_mul.cpp:48-56
     g = torch.tensor([[-3.0, -1, 0, 1], [2, 4, 0.5, -0.5]])
